@@ -1,0 +1,223 @@
+#!/usr/bin/env python3
+"""Benchmark of the ROCm memory component's reduce_multi on one MI355X.
+
+A "step" is one reduce_multi call on the headline workload: FLOAT32 SUM of 8
+source vectors of 67,108,864 elements (256 MiB each, stride 256 MiB in one
+slab) into a 9th vector -- a radix-8 k-nomial step on 256 MiB buffers.  Inputs
+are generated on the device (uniform [-1,1), seeded) and are resident in HBM
+before the timed region.  Prints ONE JSON line.
+
+  value            algorithmic GB/s over K steps: K stream-ordered launches
+                   (reduce_multi_nb through the dispatcher's C ABI) bracketed
+                   by stream synchronisation, bytes = (N+1)*size*4 per step
+  roofline         the same bytes / the kernel's average duration, measured
+                   with HIP event pairs on the component's stream around each
+                   launch, against 8 TB/s HBM3E
+  cpu_baseline     the CPU oracle (port of the reference's host fold, one
+                   thread) timed on this box on the same workload
+  latency_us       small-message p50 per call, FLOAT32 SUM, 2/4/8 sources
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+N_SRC = 8
+SIZE = 67108864
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--size", type=int, default=SIZE, help="elements per vector (default: the headline 67,108,864)")
+    ap.add_argument("--nsrc", type=int, default=N_SRC)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-latency", action="store_true", help="skip the small-message sweep")
+    ap.add_argument("--latency-iters", type=int, default=2000)
+    ap.add_argument("--latency-full", action="store_true",
+                    help="all 14 sizes x 10,000 iterations; table to gpurun_out/latency.json")
+    return ap.parse_args()
+
+
+def cpu_baseline(size, nsrc):
+    """The oracle's single-thread fold on the same workload, host memory."""
+    from oracle import pyoracle as o
+    from xccl_amd.types import Dt, Op
+    threads = max(1, min(16, os.cpu_count() or 1))
+    slab = o.slab(nsrc, size, Dt.FLOAT32, 2, threads=threads)
+    out = np.empty(size, dtype=np.float32)
+    nbytes = (nsrc + 1) * size * 4
+    stride = size * 4
+
+    def run(th):
+        t0 = time.perf_counter()
+        o.reduce_multi(slab, slab, out, nsrc - 1, size, stride, Dt.FLOAT32, Op.SUM, off2=stride, threads=th)
+        return time.perf_counter() - t0
+
+    run(1)
+    t1 = []
+    while sum(t1) < 8.0 and len(t1) < 10:
+        t1.append(run(1))
+    run(threads)
+    tm = []
+    while sum(tm) < 4.0 and len(tm) < 10:
+        tm.append(run(threads))
+    med1, medm = float(np.median(t1)), float(np.median(tm))
+    return {
+        "value": round(nbytes / med1 / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": "%d calls of the full workload (%d x %d fp32, %d B/call), median %.1f ms/call; host traffic is "
+                  "3*(N-1)*size*4 B/call" % (len(t1), nsrc, size, nbytes, med1 * 1e3),
+        "all_cores": {"value": round(nbytes / medm / 1e9, 3), "cores": threads, "ms_per_call": round(medm * 1e3, 2)},
+    }, slab, out
+
+
+def latency_sweep(mc, hip, iters, full):
+    from xccl_amd.types import Dt, MemType, Op, Status
+    sizes_b = [4 << k for k in range(14)] if full else [4, 1024, 32768]
+    if full:
+        iters = 10000
+    res = {}
+    maxb = 32768
+    buf = hip.DeviceBuffer(10 * maxb)
+    for j in range(9):
+        mc.datagen_fill(buf.ptr + j * maxb, maxb // 4, Dt.FLOAT32, 5, j)
+    hip.device_synchronize()
+    for nsrc in (2, 4, 8):
+        for b in sizes_b:
+            cnt = b // 4
+            row = {}
+            for mode in ("sync", "event", "graph"):
+                st, ns = mc.bench_latency(mode, buf.ptr, buf.ptr + maxb, buf.ptr + 9 * maxb, nsrc - 1, cnt, maxb,
+                                          Dt.FLOAT32, Op.SUM, iters)
+                assert st == Status.OK, (mode, st)
+                ns = ns[iters // 10:]
+                row[mode] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
+                             "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
+            res["n%d_%dB" % (nsrc, b)] = row
+    buf.close()
+    return res
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the reduction path is local arithmetic between p2p rounds; "
+              "no inter-GPU work exists to scale) -- use --gpus 1", file=sys.stderr)
+        return 2
+
+    from xccl_amd import hip, mc
+    from xccl_amd.types import Dt, MemType, Op, Status
+
+    if hip.device_count() < 1:
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    hip.set_device(0)
+    assert mc.xccl_mem_component_init() == Status.OK
+    assert bool(mc.dispatch_lib().xccl_mem_component_get(int(MemType.ROCM))), "ROCm component not loaded"
+
+    size, nsrc = a.size, a.nsrc
+    stride = size * 4
+    nbytes = (nsrc + 1) * size * 4
+    st, slab = mc.xccl_mem_component_alloc((nsrc + 1) * stride, MemType.ROCM)
+    assert st == Status.OK
+    dst = slab + nsrc * stride
+    for j in range(nsrc):
+        assert mc.datagen_fill(slab + j * stride, size, Dt.FLOAT32, 2, j) == Status.OK
+    hip.device_synchronize()
+    stream = mc.component_stream()
+
+    def step():
+        st_, _ = mc.xccl_mem_component_reduce_multi_nb(slab, slab + stride, dst, nsrc - 1, size, stride, Dt.FLOAT32,
+                                                       Op.SUM, MemType.ROCM, None, want_event=False)
+        assert st_ == Status.OK
+
+    for _ in range(a.warmup):
+        step()
+    hip.stream_synchronize(stream)
+    hip.device_synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    hip.stream_synchronize(stream)
+    hip.device_synchronize()
+    dt_total = time.perf_counter() - t0
+    ms_per_step = dt_total / a.steps * 1e3
+    gbps = nbytes / (dt_total / a.steps) / 1e9
+
+    # the blocking vtable entry (launch + synchronize inside), for comparison
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        assert mc.xccl_mem_component_reduce_multi(slab, slab + stride, dst, nsrc - 1, size, stride, Dt.FLOAT32, Op.SUM,
+                                                  MemType.ROCM) == Status.OK
+    sync_ms = (time.perf_counter() - t0) / a.steps * 1e3
+
+    # per-launch device time from HIP event pairs on the kernel's own stream
+    st, kms = mc.bench_kernel_times(slab, slab + stride, dst, nsrc - 1, size, stride, Dt.FLOAT32, Op.SUM,
+                                    max(a.steps, 10))
+    assert st == Status.OK
+    k_avg = float(np.mean(kms))
+    achieved = nbytes / (k_avg * 1e-3) / 1e9
+    traffic = None
+    if os.path.isfile(TRAFFIC_FILE) and size == SIZE and nsrc == N_SRC:
+        try:
+            traffic = json.load(open(TRAFFIC_FILE)).get("bytes_per_launch")
+        except Exception:
+            traffic = None
+    grid, block, name = mc._c.c_uint(0), mc._c.c_uint(0), mc._c.create_string_buffer(256)
+    mc.component_lib().xccl_rocm_reduce_multi_plan(slab, slab + stride, dst, nsrc - 1, size, stride, int(Dt.FLOAT32),
+                                                   int(Op.SUM), mc._c.byref(grid), mc._c.byref(block), name, 256)
+
+    out = {
+        "metric": "reduce_multi GB/s (fp32 sum, %d srcs x %d MiB)" % (nsrc, stride >> 20),
+        "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "reduce_multi FLOAT32 SUM, %d source vectors x %d elements at stride %d B in one slab "
+                               "(BASELINE configs[1]); stream-ordered launches" % (nsrc, size, stride),
+                   "bytes_per_step": nbytes, "device": hip.device_name(0),
+                   "kernel": name.value.decode(), "grid": grid.value, "block": block.value},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "sync_entry": {"ms_per_step": round(sync_ms, 4), "GBps": round(nbytes / sync_ms / 1e6, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(float(np.min(kms)), 4),
+                     "launches_timed": int(kms.size)},
+    }
+
+    if not a.no_cpu:
+        cb, host_slab, host_out = cpu_baseline(size, nsrc)
+        out["cpu_baseline"] = cb
+        # same inputs on both sides: the GPU result must equal the CPU fold bit for bit
+        got = np.empty(size, dtype=np.float32)
+        hip.memcpy_dtoh(got, dst)
+        out["matches_cpu_oracle"] = bool(got.tobytes() == host_out.tobytes())
+        del host_slab, host_out, got
+    else:
+        out["cpu_baseline"] = None
+
+    if not a.no_latency:
+        lat = latency_sweep(mc, hip, a.latency_iters, a.latency_full)
+        if a.latency_full:
+            os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+            json.dump(lat, open(os.path.join(ROOT, "gpurun_out", "latency.json"), "w"), indent=1)
+            out["latency_us"] = {k: v for k, v in lat.items() if k.endswith(("_4B", "_1024B", "_32768B"))}
+        else:
+            out["latency_us"] = lat
+
+    mc.xccl_mem_component_free(slab, MemType.ROCM)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,104 @@
+/*
+ * xccl_rocm_kernels.h -- the C ABI between the C host side of the ROCm
+ * memory component and its gfx950 HIP kernels.
+ *
+ * It takes the place of the two `extern "C"` launchers the reference's CUDA
+ * component declares for itself (src/utils/cuda/cuda_mem_component.c:110-125)
+ * and defines in src/utils/cuda/kernels/xccl_cuda_reduce.cu:105-133 and
+ * xccl_cuda_reduce_multi.cu:110-142.  Differences that a caller can see:
+ *
+ *   - every function here only ENQUEUES work on `hip_stream` (a hipStream_t
+ *     passed as void*; NULL is the legacy default stream).  The reference
+ *     launchers end with cudaStreamSynchronize; here waiting is the caller's
+ *     business (the component's synchronous vtable entries do it).
+ *   - `stride` is used in bytes exactly as given; it need not be a multiple
+ *     of the element size (the reference asserts that it is).
+ *   - fold order and operand order follow the reference's HOST path
+ *     (src/utils/mem_component.c:133-139): acc = OP(sbuf1, sbuf2{0}), then
+ *     acc = OP(sbuf2{j}, acc) for j = 1 .. count-1.  count == 0 behaves as
+ *     count == 1, as it does there.
+ *   - datatype coverage is INT8..INT64, UINT8..UINT64 (10 ops) and
+ *     FLOAT16/32/64 (MAX, MIN, SUM, PROD); everything else returns
+ *     XCCL_ERR_UNSUPPORTED (the reference kernels' convention).
+ *
+ * No pointer needs any alignment beyond what the caller already has; rbuf /
+ * target may be exactly equal to any one source vector (in-place), and must
+ * not overlap a source in any other way.
+ */
+#ifndef XCCL_ROCM_KERNELS_H_
+#define XCCL_ROCM_KERNELS_H_
+
+#include "xccl_rocm_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* XCCL_OK if a kernel exists for (dtype, op), XCCL_ERR_UNSUPPORTED if not.
+ * Host-only; touches no device.  Same matrix as the two launchers below. */
+xccl_status_t xccl_rocm_reduce_supported(xccl_dt_t dtype, xccl_op_t op);
+
+/* target[i] = OP(sbuf1[i], sbuf2[i]), i < count.
+ * Replaces xccl_cuda_reduce_impl (xccl_cuda_reduce.cu:105-133). */
+xccl_status_t xccl_rocm_reduce_impl(void *sbuf1, void *sbuf2, void *target,
+                                    size_t count, xccl_dt_t dtype,
+                                    xccl_op_t op, void *hip_stream);
+
+/* rbuf = sbuf1 OP sbuf2{0} OP ... OP sbuf2{count-1}; `size` elements per
+ * vector, vectors of sbuf2 `stride` bytes apart.  One kernel launch, every
+ * source read once, accumulator in registers.
+ * Replaces xccl_cuda_reduce_multi_impl (xccl_cuda_reduce_multi.cu:110-142). */
+xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf,
+                                          size_t count, size_t size,
+                                          size_t stride, xccl_dt_t dtype,
+                                          xccl_op_t op, void *hip_stream);
+
+/* Same contract and same kernel as xccl_rocm_reduce_multi_impl, but enqueued
+ * as one launch of a pre-instantiated single-kernel-node hipGraph whose node
+ * parameters are patched per call (a small per-device cache keeps the most
+ * recent argument sets instantiated, so a k-nomial step that repeats with the
+ * same buffers replays its graph untouched).  No counterpart in the
+ * reference.  Calls on one device serialise on an internal lock. */
+xccl_status_t xccl_rocm_reduce_multi_graph(void *sbuf1, void *sbuf2, void *rbuf,
+                                           size_t count, size_t size,
+                                           size_t stride, xccl_dt_t dtype,
+                                           xccl_op_t op, void *hip_stream);
+
+/* Drop every cached graph of the current device (component close). */
+void xccl_rocm_graph_cache_destroy(void);
+
+/*
+ * Launch-shape knobs, for measurement.  `blocks_per_cu` caps the persistent
+ * grid at blocks_per_cu x (compute units); 0 restores the built-in default.
+ * `nontemporal` != 0 selects kernels whose loads/stores carry the
+ * non-temporal hint.  Both are process-global and may also be set through
+ * the environment (XCCL_MC_ROCM_BLOCKS_PER_CU, XCCL_MC_ROCM_NONTEMPORAL),
+ * read once at first launch.
+ */
+void xccl_rocm_set_launch_shape(int blocks_per_cu, int nontemporal);
+
+/* What a launch with these arguments would be: grid/block size and the
+ * mangled kernel name (truncated into `name`, if not NULL).  Host-only apart
+ * from the CU-count query.  Returns the status the launch would return. */
+xccl_status_t xccl_rocm_reduce_multi_plan(void *sbuf1, void *sbuf2, void *rbuf,
+                                          size_t count, size_t size,
+                                          size_t stride, xccl_dt_t dtype,
+                                          xccl_op_t op, unsigned *grid,
+                                          unsigned *block, char *name,
+                                          size_t name_len);
+
+/*
+ * Stream gate used by start/finish_stream_activity: one wave polls the
+ * host-mapped word at `dev_flag` until it is non-zero, or until `max_ns`
+ * nanoseconds have passed (then it stores 2 to `dev_flag` itself and exits:
+ * a gate the host never opens cannot hang the queue).
+ * Replaces xccl_cuda_dummy_kernel (xccl_cuda_kernel.cu:4-20), which spins
+ * without a bound.
+ */
+xccl_status_t xccl_rocm_stream_gate(int *dev_flag, uint64_t max_ns,
+                                    void *hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XCCL_ROCM_KERNELS_H_ */

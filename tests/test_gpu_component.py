@@ -1,0 +1,247 @@
+"""The rest of the component's vtable on a real device: memory-type probing,
+the dispatcher's buffer cache on device memory, events and their pool,
+stream-ordered reductions, the graph launch path, the stream gate, and the
+synthetic-input kernels against the oracle's generator."""
+import ctypes
+import time
+
+import numpy as np
+import pytest
+
+from gpu_util import NP, Case, assert_same
+from xccl_amd import hip
+from xccl_amd.types import Dt, MemType, Op, Status, StreamType, dt_size
+
+pytestmark = pytest.mark.gpu
+
+
+def test_mem_type_probe(rocm):
+    """cuda_mem_component.c:182-204: device memory -> the component's type,
+    pinned host memory -> HOST, ordinary host memory -> HOST (component says
+    UNSUPPORTED, dispatcher falls through), and the runtime is left without a
+    sticky error."""
+    d = hip.DeviceBuffer(1024)
+    assert rocm.xccl_mem_component_type(d.ptr) == (Status.OK, MemType.ROCM)
+    assert rocm.xccl_mem_component_type(d.ptr + 512) == (Status.OK, MemType.ROCM)
+    pinned = hip.host_malloc(1024)
+    assert rocm.xccl_mem_component_type(pinned) == (Status.OK, MemType.HOST)
+    plain = ctypes.create_string_buffer(64)
+    assert rocm.xccl_mem_component_type(ctypes.addressof(plain)) == (Status.OK, MemType.HOST)
+    mt = ctypes.c_int(-1)
+    st = rocm.component().super.mem_type(ctypes.addressof(plain), ctypes.byref(mt))
+    assert st in (Status.ERR_UNSUPPORTED, Status.OK)
+    assert hip.lib().hipGetLastError() == 0
+    hip.host_free(pinned)
+    d.close()
+
+
+def test_device_alloc_cache(rocm):
+    """mem_component.c:51-105 on the real component: a request that fits the
+    4 KiB cache gets the cached device buffer, a second concurrent one and an
+    oversized one get their own."""
+    st, p1 = rocm.xccl_mem_component_alloc(3 * 1024, MemType.ROCM)
+    assert st == Status.OK and rocm.xccl_mem_component_type(p1) == (Status.OK, MemType.ROCM)
+    st, p2 = rocm.xccl_mem_component_alloc(3 * 1024, MemType.ROCM)
+    assert st == Status.OK and p2 != p1
+    assert rocm.xccl_mem_component_free(p1, MemType.ROCM) == Status.OK
+    st, p3 = rocm.xccl_mem_component_alloc(4096, MemType.ROCM)
+    assert p3 == p1
+    st, p4 = rocm.xccl_mem_component_alloc(1 << 20, MemType.ROCM)
+    assert st == Status.OK and p4 not in (p1, p2)
+    for p in (p2, p3, p4):
+        assert rocm.xccl_mem_component_free(p, MemType.ROCM) == Status.OK
+
+
+def test_event_record_query_free_and_pool(rocm):
+    """Pool exhaustion is XCCL_ERR_NO_RESOURCE (cuda_mem_component.c:91,107);
+    a freed slot is reusable."""
+    s = rocm.Stream(hip.stream_create())
+    evs = []
+    while True:
+        st, ev = rocm.xccl_mc_event_record(s)
+        if st != Status.OK:
+            break
+        evs.append(ev)
+        assert len(evs) <= 4096
+    assert st == Status.ERR_NO_RESOURCE and len(evs) == 64
+    hip.stream_synchronize(s.hip_stream)
+    for ev in evs:
+        assert ctypes.c_int.from_address(ev).value == MemType.ROCM
+        assert rocm.xccl_mc_event_query(ev) == Status.OK
+        assert rocm.xccl_mc_event_free(ev) == Status.OK
+    st, ev = rocm.xccl_mc_event_record(s)
+    assert st == Status.OK
+    assert rocm.xccl_mc_event_wait(ev) == Status.OK
+    assert rocm.xccl_mc_event_free(ev) == Status.OK
+    hip.stream_destroy(s.hip_stream)
+
+
+@pytest.mark.parametrize("own_stream", [False, True])
+def test_stream_ordered_reduce_multi(rocm, oracle, own_stream):
+    """reduce_multi_nb returns with the kernel enqueued; the event turns from
+    INPROGRESS/OK to OK and the result is then complete.  Two dependent calls
+    on one stream (round k's rbuf is round k+1's sbuf1, allreduce_knomial.c:
+    118-135) need no host wait in between."""
+    dt, op, size, n2 = Dt.FLOAT32, Op.SUM, 1 << 22, 3
+    c = Case(dt, size, n2)
+    s = rocm.Stream(hip.stream_create()) if own_stream else None
+    try:
+        c.fill_random(oracle, 12)
+        c.upload()
+        p1, p2, pr = c.ptrs()
+        st, ev1 = rocm.xccl_mem_component_reduce_multi_nb(p1, p2, pr, n2, size, c.stride, dt, op, MemType.ROCM, s)
+        assert st == Status.OK and ev1
+        st, ev2 = rocm.xccl_mem_component_reduce_multi_nb(pr, p2, pr, n2, size, c.stride, dt, op, MemType.ROCM, s)
+        assert st == Status.OK and ev2
+        t0 = time.time()
+        while True:
+            q = rocm.xccl_mc_event_query(ev2)
+            if q == Status.OK:
+                break
+            assert q == Status.INPROGRESS and time.time() - t0 < 30
+        assert rocm.xccl_mc_event_query(ev1) == Status.OK
+        img = c.host.copy()
+        b = img.ctypes.data
+        oracle.reduce_multi_ptr(b + c.o1, b + c.o2, b + c.orr, n2, size, c.stride, dt, op)
+        oracle.reduce_multi_ptr(b + c.orr, b + c.o2, b + c.orr, n2, size, c.stride, dt, op)
+        assert_same(c.result(), img[c.orr: c.orr + c.vbytes], dt, op, "nb chain")
+        assert rocm.xccl_mc_event_free(ev1) == Status.OK and rocm.xccl_mc_event_free(ev2) == Status.OK
+        # without an event: completion through the stream itself
+        st, ev = rocm.xccl_mem_component_reduce_nb(p1, p2, pr, size, dt, op, MemType.ROCM, s, want_event=False)
+        assert st == Status.OK and not ev
+        hip.stream_synchronize(s.hip_stream if s else rocm.component_stream())
+        want = np.empty(size, dtype=np.float32)
+        oracle.dt_reduce(c.host[c.o1:c.o1 + c.vbytes].view(np.float32), c.host[c.o2:c.o2 + c.vbytes].view(np.float32),
+                         want, size, dt, op)
+        assert_same(c.result(), want.view(np.uint8), dt, op, "reduce_nb")
+        # unsupported pair: status, no event consumed
+        st, ev = rocm.xccl_mem_component_reduce_multi_nb(p1, p2, pr, n2, size, c.stride, dt, Op.BAND, MemType.ROCM, s)
+        assert st == Status.ERR_UNSUPPORTED and not ev
+    finally:
+        c.close()
+        if s:
+            hip.stream_destroy(s.hip_stream)
+
+
+def test_graph_launch_matches_plain_launch(rocm, oracle):
+    """The single-node graph path: same bits as the plain launch, across cache
+    hits (same arguments replayed), parameter patches (more argument sets than
+    cache slots) and several replays with other work in between."""
+    lib = rocm.component_lib()
+    stream = rocm.component_stream()
+    dt, op = Dt.FLOAT32, Op.SUM
+    cases = []
+    try:
+        for k in range(11):                      # > 8 cache slots
+            c = Case(dt, 64 + 257 * k, 1 + k % 4, off2=4 * (k % 3))
+            c.fill_random(oracle, 30 + k)
+            c.upload()
+            cases.append(c)
+        for rep in range(3):
+            for c in cases:
+                p1, p2, pr = c.ptrs()
+                hip.memset(pr, 0xEE, c.vbytes)
+                st = lib.xccl_rocm_reduce_multi_graph(p1, p2, pr, c.n2, c.size, c.stride, int(dt), int(op), stream)
+                assert st == Status.OK
+                if rep == 1:                     # immediate replay: cache hit
+                    assert lib.xccl_rocm_reduce_multi_graph(p1, p2, pr, c.n2, c.size, c.stride, int(dt), int(op),
+                                                            stream) == Status.OK
+                hip.stream_synchronize(stream)
+                want, _ = c.expect(oracle, op)
+                assert_same(c.result(), want, dt, op, "graph rep %d size %d" % (rep, c.size))
+            # eager work between rounds of replays
+            run = cases[0]
+            p1, p2, pr = run.ptrs()
+            assert rocm.xccl_mem_component_reduce_multi(p1, p2, pr, run.n2, run.size, run.stride, dt, op,
+                                                        MemType.ROCM) == Status.OK
+        assert lib.xccl_rocm_reduce_multi_graph(p1, p2, pr, 1, 16, 64, int(dt), int(Op.BAND), stream) \
+            == Status.ERR_UNSUPPORTED
+    finally:
+        for c in cases:
+            c.close()
+        lib.xccl_rocm_graph_cache_destroy()
+
+
+def test_memcpy_async_source_first(rocm):
+    """mem_component.h:38: (sbuf, dbuf, size, stream) -- source first."""
+    s = rocm.Stream(hip.stream_create())
+    a = hip.DeviceBuffer(4096)
+    b = hip.DeviceBuffer(4096)
+    data = np.arange(1024, dtype=np.uint32)
+    a.upload(data)
+    hip.memset(b.ptr, 0, 4096)
+    assert rocm.xccl_mem_component_memcpy_async(a.ptr, b.ptr, 4096, s) == Status.OK
+    hip.stream_synchronize(s.hip_stream)
+    assert np.array_equal(b.download(np.uint32, 1024), data)
+    hip.stream_destroy(s.hip_stream)
+    a.close()
+    b.close()
+
+
+def test_stream_activity_gate(rocm):
+    """cuda_mem_component.c:139-180: work enqueued on the user stream after
+    start_stream_activity does not run until finish_stream_activity.  The gate
+    kernel's wait is bounded, so nothing here can hang the queue."""
+    s = rocm.Stream(hip.stream_create())
+    a = hip.DeviceBuffer(4096)
+    b = hip.DeviceBuffer(4096)
+    a.upload(np.full(1024, 7, dtype=np.uint32))
+    hip.memset(b.ptr, 0, 4096)
+    st, req = rocm.xccl_mem_component_start_acitivity(s)
+    assert st == Status.OK and ctypes.c_int.from_address(req).value == MemType.ROCM
+    assert rocm.xccl_mem_component_memcpy_async(a.ptr, b.ptr, 4096, s) == Status.OK
+    st, ev = rocm.xccl_mc_event_record(s)
+    assert st == Status.OK
+    time.sleep(0.2)
+    assert rocm.xccl_mc_event_query(ev) == Status.INPROGRESS      # still gated
+    assert rocm.xccl_mem_component_finish_acitivity(req) == Status.OK
+    assert rocm.xccl_mc_event_wait(ev) == Status.OK
+    assert (b.download(np.uint32, 1024) == 7).all()
+    assert rocm.xccl_mc_event_free(ev) == Status.OK
+    # slots recycle: more start/finish pairs than the pool holds
+    for _ in range(10):
+        st, req = rocm.xccl_mem_component_start_acitivity(s)
+        assert st == Status.OK
+        assert rocm.xccl_mem_component_finish_acitivity(req) == Status.OK
+        hip.stream_synchronize(s.hip_stream)
+    hip.stream_destroy(s.hip_stream)
+    a.close()
+    b.close()
+
+
+def test_stream_gate_times_out_by_itself(rocm):
+    """A gate nobody opens leaves after its time limit and marks the word with
+    2 (forced from the host with a 50 ms limit; no wave is left spinning)."""
+    lib = rocm.component_lib()
+    flag_host = hip.host_malloc(64)
+    ctypes.c_int.from_address(flag_host).value = 0
+    dev = ctypes.c_void_p()
+    hip.check(hip.lib().hipHostGetDevicePointer(ctypes.byref(dev), ctypes.c_void_p(flag_host), 0))
+    stream = rocm.component_stream()
+    t0 = time.time()
+    assert lib.xccl_rocm_stream_gate(dev, 50 * 1000 * 1000, stream) == Status.OK
+    hip.stream_synchronize(stream)
+    dt = time.time() - t0
+    assert ctypes.c_int.from_address(flag_host).value == 2
+    assert 0.03 < dt < 5.0
+    hip.host_free(flag_host)
+
+
+@pytest.mark.parametrize("dt", [Dt.INT8, Dt.UINT16, Dt.INT32, Dt.UINT64, Dt.FLOAT16, Dt.FLOAT32, Dt.FLOAT64],
+                         ids=lambda d: Dt(d).name)
+def test_datagen_matches_oracle_generator(rocm, oracle, dt):
+    """The GPU input generator and the oracle's CPU generator follow one
+    recipe: identical bits for integers, binary16 and binary32; binary64 goes
+    through log/cos of two different math libraries and agrees to 1e-13."""
+    n = 100003
+    d = hip.DeviceBuffer(n * dt_size(dt))
+    for sparse in (False, True):
+        assert rocm.datagen_fill(d.ptr, n, dt, 5, 3, sparse) == Status.OK
+        hip.device_synchronize()
+        got = d.download(NP[int(dt)], n)
+        want = oracle.fill(n, dt, 5, 3, sparse)
+        if dt == Dt.FLOAT64:
+            assert np.allclose(got, want, rtol=0, atol=1e-13)
+        else:
+            assert got.tobytes() == want.tobytes()
+    d.close()

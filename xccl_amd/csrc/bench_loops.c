@@ -1,0 +1,112 @@
+/*
+ * bench_loops.c -- timing loops for the small-message latency sweep, in C so
+ * that the per-call figure holds no interpreter overhead.  Part of
+ * libxccl_rocm_benchkit.so (bench and tests only; not loaded by the
+ * component).  The component is reached through the pointer the caller
+ * passes, i.e. through the same exported object libxccl would use.
+ */
+#include "xccl_rocm_kernels.h"
+#include "xccl_rocm_mem_component.h"
+
+#include <hip/hip_runtime_api.h>
+#include <time.h>
+
+static inline uint64_t now_ns(void)
+{
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (uint64_t)ts.tv_sec * 1000000000ull + (uint64_t)ts.tv_nsec;
+}
+
+typedef xccl_status_t (*graph_fn_t)(void *, void *, void *, size_t, size_t, size_t, xccl_dt_t, xccl_op_t, void *);
+
+/*
+ * Runs `iters` back-to-back reduce_multi calls and stores each call's
+ * host-observed duration (entry to completion seen by the host) in ns_out.
+ *   mode 0: the synchronous vtable entry (launch + stream synchronize inside)
+ *   mode 1: reduce_multi_nb on the component stream + event_query polling
+ *   mode 2: `graph_fn` (xccl_rocm_reduce_multi_graph) + hipStreamSynchronize
+ *   mode 3: reduce_multi_nb without event + hipStreamSynchronize
+ * Returns the first non-OK status, or XCCL_OK.
+ */
+xccl_status_t xccl_rocm_bench_latency(xccl_rocm_mem_component_t *mc, graph_fn_t graph_fn, int mode, void *sbuf1,
+                                      void *sbuf2, void *rbuf, size_t count, size_t size, size_t stride,
+                                      xccl_dt_t dtype, xccl_op_t op, size_t iters, uint64_t *ns_out)
+{
+    void         *stream = NULL;
+    xccl_status_t st     = mc->get_stream(&stream);
+    size_t        i;
+
+    if (st != XCCL_OK) {
+        return st;
+    }
+    for (i = 0; i < iters; i++) {
+        const uint64_t t0 = now_ns();
+        if (mode == 0) {
+            st = mc->super.reduce_multi(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op);
+        } else if (mode == 1) {
+            xccl_mc_event_t *ev = NULL;
+            st = mc->reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, NULL, &ev);
+            if (st == XCCL_OK) {
+                while ((st = mc->super.event_query(ev)) == XCCL_INPROGRESS) {
+                }
+                mc->super.event_free(ev);
+            }
+        } else if (mode == 2) {
+            st = graph_fn(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, stream);
+            if (st == XCCL_OK && hipStreamSynchronize((hipStream_t)stream) != hipSuccess) {
+                st = XCCL_ERR_NO_MESSAGE;
+            }
+        } else {
+            st = mc->reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, NULL, NULL);
+            if (st == XCCL_OK && hipStreamSynchronize((hipStream_t)stream) != hipSuccess) {
+                st = XCCL_ERR_NO_MESSAGE;
+            }
+        }
+        ns_out[i] = now_ns() - t0;
+        if (st != XCCL_OK) {
+            return st;
+        }
+    }
+    return XCCL_OK;
+}
+
+/*
+ * Enqueues `iters` stream-ordered reduce_multi calls back to back on the
+ * component stream, each bracketed by its own pair of timing events, waits
+ * once, and stores each launch's device-side duration in ms_out.  `ev` holds
+ * 2*iters timing-enabled hipEvent_t created by the caller.
+ */
+xccl_status_t xccl_rocm_bench_kernel_times(xccl_rocm_mem_component_t *mc, void *sbuf1, void *sbuf2, void *rbuf,
+                                           size_t count, size_t size, size_t stride, xccl_dt_t dtype, xccl_op_t op,
+                                           size_t iters, void **ev, float *ms_out)
+{
+    void         *stream = NULL;
+    xccl_status_t st     = mc->get_stream(&stream);
+    size_t        i;
+
+    if (st != XCCL_OK) {
+        return st;
+    }
+    for (i = 0; i < iters; i++) {
+        if (hipEventRecord((hipEvent_t)ev[2 * i], (hipStream_t)stream) != hipSuccess) {
+            return XCCL_ERR_NO_MESSAGE;
+        }
+        st = mc->reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, NULL, NULL);
+        if (st != XCCL_OK) {
+            return st;
+        }
+        if (hipEventRecord((hipEvent_t)ev[2 * i + 1], (hipStream_t)stream) != hipSuccess) {
+            return XCCL_ERR_NO_MESSAGE;
+        }
+    }
+    if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) {
+        return XCCL_ERR_NO_MESSAGE;
+    }
+    for (i = 0; i < iters; i++) {
+        if (hipEventElapsedTime(&ms_out[i], (hipEvent_t)ev[2 * i], (hipEvent_t)ev[2 * i + 1]) != hipSuccess) {
+            return XCCL_ERR_NO_MESSAGE;
+        }
+    }
+    return XCCL_OK;
+}

@@ -1,0 +1,101 @@
+// datagen.hip -- libxccl_rocm_benchkit.so: fills device buffers with the
+// synthetic workload of the benchmarks, on the GPU.  Not part of the memory
+// component; bench and tests use it so that multi-GiB inputs need not cross
+// PCIe.
+//
+// Every element is a pure function of (seed, vector index, element index):
+//     x = splitmix64(seed * 0x9E3779B97F4A7C15 + (vec << 40) + i)
+//     FLOAT32  (x >> 40) * 2^-23 - 1          uniform [-1, 1), exact
+//     FLOAT16  (x >> 53) * 2^-11 - 0.5        uniform [-0.5, 0.5), exact
+//     FLOAT64  Box-Muller normal(0, 1) from x and y = splitmix64(x)
+//     integers the low 8*sizeof(T) bits of x (full range); with `sparse`
+//              set, the element is zeroed when bit 63 of y is set (the
+//              inputs of the logical operators: half zeros)
+// The CPU generator of the test oracle follows the same recipe; the two agree
+// bit for bit except FLOAT64, where log/cos come from different math
+// libraries.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "xccl_rocm_types.h"
+
+namespace {
+
+__host__ __device__ inline uint64_t splitmix64(uint64_t z)
+{
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+template <typename T> struct Gen;
+
+template <> struct Gen<float> {
+    static __device__ float make(uint64_t x, uint64_t, int) { return (float)(x >> 40) * 0x1p-23f - 1.0f; }
+};
+template <> struct Gen<_Float16> {
+    static __device__ _Float16 make(uint64_t x, uint64_t, int) { return (_Float16)((float)(x >> 53) * 0x1p-11f - 0.5f); }
+};
+template <> struct Gen<double> {
+    static __device__ double make(uint64_t x, uint64_t y, int)
+    {
+        const double u1 = ((double)(x >> 11) + 1.0) * 0x1p-53; // (0, 1]
+        const double u2 = (double)(y >> 11) * 0x1p-53;         // [0, 1)
+        return sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2);
+    }
+};
+template <typename T> struct Gen {
+    static __device__ T make(uint64_t x, uint64_t y, int sparse) { return (sparse && (y >> 63)) ? (T)0 : (T)x; }
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) fill_kernel(T *dst, size_t count, uint64_t base, int sparse)
+{
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += step) {
+        const uint64_t x = splitmix64(base + i);
+        dst[i]           = Gen<T>::make(x, splitmix64(x), sparse);
+    }
+}
+
+template <typename T>
+hipError_t fill(void *dst, size_t count, uint64_t base, int sparse, hipStream_t s)
+{
+    size_t blocks = (count + 255) / 256;
+    if (blocks > 65536) {
+        blocks = 65536;
+    }
+    hipLaunchKernelGGL(fill_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, (T *)dst, count, base, sparse);
+    return hipGetLastError();
+}
+
+} // namespace
+
+// Fills dst[0 .. count) with vector `vec` of the stream identified by `seed`.
+// Enqueues on `hip_stream` (hipStream_t as void*) and returns.
+extern "C" xccl_status_t xccl_rocm_datagen_fill(void *dst, size_t count, xccl_dt_t dtype, uint64_t seed, uint64_t vec,
+                                                int sparse, void *hip_stream)
+{
+    const uint64_t base = seed * 0x9E3779B97F4A7C15ull + (vec << 40);
+    hipStream_t    s    = (hipStream_t)hip_stream;
+    hipError_t     e;
+    if (count == 0) {
+        return XCCL_OK;
+    }
+    switch (dtype) {
+    case XCCL_DT_INT8:
+    case XCCL_DT_UINT8:   e = fill<uint8_t>(dst, count, base, sparse, s); break;
+    case XCCL_DT_INT16:
+    case XCCL_DT_UINT16:  e = fill<uint16_t>(dst, count, base, sparse, s); break;
+    case XCCL_DT_INT32:
+    case XCCL_DT_UINT32:  e = fill<uint32_t>(dst, count, base, sparse, s); break;
+    case XCCL_DT_INT64:
+    case XCCL_DT_UINT64:  e = fill<uint64_t>(dst, count, base, sparse, s); break;
+    case XCCL_DT_FLOAT16: e = fill<_Float16>(dst, count, base, sparse, s); break;
+    case XCCL_DT_FLOAT32: e = fill<float>(dst, count, base, sparse, s); break;
+    case XCCL_DT_FLOAT64: e = fill<double>(dst, count, base, sparse, s); break;
+    default:              return XCCL_ERR_UNSUPPORTED;
+    }
+    return e == hipSuccess ? XCCL_OK : XCCL_ERR_NO_MESSAGE;
+}

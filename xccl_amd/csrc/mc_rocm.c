@@ -1,0 +1,536 @@
+/*
+ * mc_rocm.c -- the ROCm memory component of XCCL: the object that
+ * xccl_rocm_mem_component.so exports and libxccl's mem-component dispatcher
+ * calls through (vtable: reference src/utils/mem_component.h:28-49).
+ *
+ * It stands where the reference's CUDA component stands
+ * (src/utils/cuda/cuda_mem_component.c) and keeps that component's contract:
+ * per-process singletons, resources created on first use (open() runs inside
+ * libxccl's ELF constructor, before the application picked a device --
+ * cuda_mem_component.c:18-32), synchronous reduce / reduce_multi, pooled
+ * events and stream requests, XCCL_ERR_NO_MESSAGE for runtime failures,
+ * XCCL_ERR_NO_RESOURCE for an empty pool, XCCL_ERR_UNSUPPORTED for a
+ * (dtype, op) without a kernel.  It differs where the reference is unsafe or
+ * slow:
+ *   - resources are kept per device ordinal, and pool slots are claimed with
+ *     atomics (the ucx team library advertises XCCL_THREAD_MODE_MULTIPLE,
+ *     src/team_lib/ucx/xccl_ucx_lib.c:631-632);
+ *   - events are created once (the reference re-creates one on every record,
+ *     cuda_mem_component.c:220, and leaks the old one);
+ *   - small synchronous reductions go out as one hipGraph launch;
+ *   - the vtable is extended with stream-ordered reductions whose completion
+ *     is an event (see include/xccl_rocm_mem_component.h).
+ *
+ * Plain C on the HIP runtime's C API; the kernels are reached through
+ * include/xccl_rocm_kernels.h only.
+ */
+#include "xccl_rocm_kernels.h"
+#include "xccl_rocm_mem_component.h"
+
+#include <hip/hip_runtime_api.h>
+#include <pthread.h>
+#include <stdatomic.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define MC_MAX_DEVICES 64
+
+/* Synchronous reductions of at most this many bytes per vector are launched
+ * through the graph path (XCCL_MC_ROCM_GRAPH_MAX_BYTES overrides; 0 = never). */
+#define MC_DEFAULT_GRAPH_MAX_BYTES 0
+
+/* Upper bound on how long a stream gate keeps a user stream blocked when
+ * finish_stream_activity is never called (XCCL_MC_ROCM_GATE_TIMEOUT_MS). */
+#define MC_DEFAULT_GATE_TIMEOUT_MS 30000
+
+/* pool slot states (`is_free` keeps the reference's member name) */
+enum { MC_SLOT_BUSY = 0, MC_SLOT_FREE = 1, MC_SLOT_DRAINING = 2 };
+
+typedef struct mc_rocm_event {
+    xccl_mc_event_t super;
+    atomic_int      is_free;
+    hipEvent_t      hip_event;
+} mc_rocm_event_t;
+
+typedef struct mc_rocm_stream_request {
+    xccl_mem_component_stream_request_t super;
+    atomic_int                          is_free;
+    int                                *flag;     /* host view of the gate word */
+    int                                *dev_flag; /* device view of the same word */
+    hipEvent_t                          hip_event;
+} mc_rocm_stream_request_t;
+
+typedef struct mc_rocm_device {
+    atomic_int               ready; /* 0 = untouched, 1 = usable */
+    hipStream_t              stream;
+    int                     *gate_words; /* pinned, mapped */
+    mc_rocm_event_t          events[XCCL_ROCM_MC_NUM_EVENTS];
+    mc_rocm_stream_request_t requests[XCCL_ROCM_MC_NUM_STREAM_REQUESTS];
+} mc_rocm_device_t;
+
+static mc_rocm_device_t mc_devices[MC_MAX_DEVICES];
+static pthread_mutex_t  mc_init_lock = PTHREAD_MUTEX_INITIALIZER;
+static size_t           mc_graph_max_bytes;
+static uint64_t         mc_gate_timeout_ns;
+
+#define MC_HIP(call)                                                              \
+    do {                                                                          \
+        hipError_t e_ = (call);                                                   \
+        if (e_ != hipSuccess && e_ != hipErrorDeinitialized) {                    \
+            fprintf(stderr, "xccl mc_rocm: %s failed with %d (%s)\n", #call,      \
+                    (int)e_, hipGetErrorString(e_));                              \
+            return XCCL_ERR_NO_MESSAGE;                                           \
+        }                                                                         \
+    } while (0)
+
+static xccl_status_t mc_rocm_open(void)
+{
+    const char *s;
+
+    /* No device call here: the process may not have chosen its GPU yet. */
+    mc_graph_max_bytes = MC_DEFAULT_GRAPH_MAX_BYTES;
+    s = getenv("XCCL_MC_ROCM_GRAPH_MAX_BYTES");
+    if (s != NULL) {
+        mc_graph_max_bytes = (size_t)strtoull(s, NULL, 0);
+    }
+    mc_gate_timeout_ns = (uint64_t)MC_DEFAULT_GATE_TIMEOUT_MS * 1000000ull;
+    s = getenv("XCCL_MC_ROCM_GATE_TIMEOUT_MS");
+    if (s != NULL) {
+        mc_gate_timeout_ns = strtoull(s, NULL, 0) * 1000000ull;
+    }
+    return XCCL_OK;
+}
+
+/* Stream, events and gate words of one device; caller holds mc_init_lock. */
+static xccl_status_t mc_rocm_device_create(mc_rocm_device_t *d)
+{
+    int i;
+
+    MC_HIP(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
+    MC_HIP(hipHostMalloc((void **)&d->gate_words,
+                         XCCL_ROCM_MC_NUM_STREAM_REQUESTS * sizeof(int),
+                         hipHostMallocMapped));
+    for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS; i++) {
+        mc_rocm_stream_request_t *r = &d->requests[i];
+        r->flag = &d->gate_words[i];
+        MC_HIP(hipHostGetDevicePointer((void **)&r->dev_flag, r->flag, 0));
+        MC_HIP(hipEventCreateWithFlags(&r->hip_event, hipEventDisableTiming));
+        atomic_store(&r->is_free, 1);
+    }
+    for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
+        MC_HIP(hipEventCreateWithFlags(&d->events[i].hip_event,
+                                       hipEventDisableTiming));
+        atomic_store(&d->events[i].is_free, 1);
+    }
+    return XCCL_OK;
+}
+
+/* The current device's resources, created on first use. */
+static xccl_status_t mc_rocm_device(mc_rocm_device_t **out)
+{
+    int               dev = 0;
+    mc_rocm_device_t *d;
+    xccl_status_t     st = XCCL_OK;
+
+    MC_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MC_MAX_DEVICES) {
+        return XCCL_ERR_NO_RESOURCE;
+    }
+    d = &mc_devices[dev];
+    if (atomic_load_explicit(&d->ready, memory_order_acquire) == 0) {
+        pthread_mutex_lock(&mc_init_lock);
+        if (atomic_load_explicit(&d->ready, memory_order_relaxed) == 0) {
+            st = mc_rocm_device_create(d);
+            if (st == XCCL_OK) {
+                atomic_store_explicit(&d->ready, 1, memory_order_release);
+            }
+        }
+        pthread_mutex_unlock(&mc_init_lock);
+    }
+    *out = d;
+    return st;
+}
+
+static xccl_status_t mc_rocm_mem_alloc(void **ptr, size_t len)
+{
+    MC_HIP(hipMalloc(ptr, len));
+    return XCCL_OK;
+}
+
+static xccl_status_t mc_rocm_mem_free(void *ptr)
+{
+    MC_HIP(hipFree(ptr));
+    return XCCL_OK;
+}
+
+/* cuda_mem_component.c:182-204: device memory -> this component's type,
+ * every other pointer the runtime knows (pinned host, managed) -> HOST, a
+ * pointer it does not know -> XCCL_ERR_UNSUPPORTED with the runtime's sticky
+ * error cleared. */
+static xccl_status_t mc_rocm_mem_type(void *ptr, ucs_memory_type_t *mem_type)
+{
+    hipPointerAttribute_t attr;
+    hipError_t            err;
+
+    err = hipPointerGetAttributes(&attr, ptr);
+    if (err != hipSuccess) {
+        (void)hipGetLastError();
+        return XCCL_ERR_UNSUPPORTED;
+    }
+    if (attr.type == hipMemoryTypeDevice) {
+        *mem_type = UCS_MEMORY_TYPE_ROCM;
+    } else {
+        *mem_type = UCS_MEMORY_TYPE_HOST;
+    }
+    return XCCL_OK;
+}
+
+static mc_rocm_event_t *mc_rocm_claim_event(mc_rocm_device_t *d)
+{
+    int i, expect;
+
+    for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
+        expect = 1;
+        if (atomic_compare_exchange_strong(&d->events[i].is_free, &expect, 0)) {
+            return &d->events[i];
+        }
+    }
+    return NULL;
+}
+
+static xccl_status_t mc_rocm_user_stream(xccl_stream_t *stream, hipStream_t *out)
+{
+    if (stream == NULL || stream->stream == NULL) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    *out = *(hipStream_t *)stream->stream;
+    return XCCL_OK;
+}
+
+/* Shared tail of the four reduction entries.  `want_sync`: block until the
+ * result is visible (the vtable's reduce / reduce_multi contract, reference
+ * xccl_cuda_reduce_multi.cu:140). */
+static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
+                                             void *rbuf, size_t count,
+                                             size_t size, size_t stride,
+                                             xccl_dt_t dtype, xccl_op_t op,
+                                             xccl_stream_t *stream,
+                                             xccl_mc_event_t **event,
+                                             int want_sync)
+{
+    mc_rocm_device_t *d;
+    mc_rocm_event_t  *ev = NULL;
+    hipStream_t       hs;
+    xccl_status_t     st;
+
+    st = xccl_rocm_reduce_supported(dtype, op);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    st = mc_rocm_device(&d);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    hs = d->stream;
+    if (stream != NULL) {
+        st = mc_rocm_user_stream(stream, &hs);
+        if (st != XCCL_OK) {
+            return st;
+        }
+    }
+    if (event != NULL) {
+        ev = mc_rocm_claim_event(d);
+        if (ev == NULL) {
+            return XCCL_ERR_NO_RESOURCE;
+        }
+    }
+
+    if (want_sync && size * xccl_dt_size(dtype) <= mc_graph_max_bytes) {
+        st = xccl_rocm_reduce_multi_graph(sbuf1, sbuf2, rbuf, count, size,
+                                          stride, dtype, op, hs);
+    } else {
+        st = xccl_rocm_reduce_multi_impl(sbuf1, sbuf2, rbuf, count, size,
+                                         stride, dtype, op, hs);
+    }
+    if (st != XCCL_OK) {
+        if (ev != NULL) {
+            atomic_store(&ev->is_free, 1);
+        }
+        return st;
+    }
+    if (ev != NULL) {
+        hipError_t e = hipEventRecord(ev->hip_event, hs);
+        if (e != hipSuccess) {
+            atomic_store(&ev->is_free, 1);
+            return XCCL_ERR_NO_MESSAGE;
+        }
+        ev->super.mem_type = UCS_MEMORY_TYPE_ROCM;
+        *event             = &ev->super;
+    }
+    if (want_sync) {
+        MC_HIP(hipStreamSynchronize(hs));
+    }
+    return XCCL_OK;
+}
+
+static xccl_status_t mc_rocm_reduce(void *sbuf1, void *sbuf2, void *target,
+                                    size_t count, xccl_dt_t dtype, xccl_op_t op)
+{
+    return mc_rocm_do_reduce_multi(sbuf1, sbuf2, target, 1, count, 0, dtype, op,
+                                   NULL, NULL, 1);
+}
+
+static xccl_status_t mc_rocm_reduce_multi(void *sbuf1, void *sbuf2, void *rbuf,
+                                          size_t count, size_t size,
+                                          size_t stride, xccl_dt_t dtype,
+                                          xccl_op_t op)
+{
+    return mc_rocm_do_reduce_multi(sbuf1, sbuf2, rbuf, count, size, stride,
+                                   dtype, op, NULL, NULL, 1);
+}
+
+static xccl_status_t mc_rocm_reduce_nb(void *sbuf1, void *sbuf2, void *target,
+                                       size_t count, xccl_dt_t dtype,
+                                       xccl_op_t op, xccl_stream_t *stream,
+                                       xccl_mc_event_t **event)
+{
+    return mc_rocm_do_reduce_multi(sbuf1, sbuf2, target, 1, count, 0, dtype, op,
+                                   stream, event, 0);
+}
+
+static xccl_status_t mc_rocm_reduce_multi_nb(void *sbuf1, void *sbuf2,
+                                             void *rbuf, size_t count,
+                                             size_t size, size_t stride,
+                                             xccl_dt_t dtype, xccl_op_t op,
+                                             xccl_stream_t *stream,
+                                             xccl_mc_event_t **event)
+{
+    return mc_rocm_do_reduce_multi(sbuf1, sbuf2, rbuf, count, size, stride,
+                                   dtype, op, stream, event, 0);
+}
+
+/* Note the argument order: source first (mem_component.h:38). */
+static xccl_status_t mc_rocm_memcpy_async(void *sbuf, void *dbuf, size_t size,
+                                          xccl_stream_t *stream)
+{
+    hipStream_t   hs;
+    xccl_status_t st = mc_rocm_user_stream(stream, &hs);
+
+    if (st != XCCL_OK) {
+        return st;
+    }
+    MC_HIP(hipMemcpyAsync(dbuf, sbuf, size, hipMemcpyDefault, hs));
+    return XCCL_OK;
+}
+
+static xccl_status_t mc_rocm_event_record(xccl_stream_t *stream,
+                                          xccl_mc_event_t **event)
+{
+    mc_rocm_device_t *d;
+    mc_rocm_event_t  *ev;
+    hipStream_t       hs;
+    hipError_t        e;
+    xccl_status_t     st;
+
+    st = mc_rocm_user_stream(stream, &hs);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    st = mc_rocm_device(&d);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    ev = mc_rocm_claim_event(d);
+    if (ev == NULL) {
+        return XCCL_ERR_NO_RESOURCE;
+    }
+    e = hipEventRecord(ev->hip_event, hs);
+    if (e != hipSuccess) {
+        atomic_store(&ev->is_free, 1);
+        return XCCL_ERR_NO_MESSAGE;
+    }
+    ev->super.mem_type = UCS_MEMORY_TYPE_ROCM;
+    *event             = &ev->super;
+    return XCCL_OK;
+}
+
+static mc_rocm_event_t *mc_rocm_event_of(xccl_mc_event_t *event)
+{
+    return (mc_rocm_event_t *)((char *)event - offsetof(mc_rocm_event_t, super));
+}
+
+static xccl_status_t mc_rocm_event_query(xccl_mc_event_t *event)
+{
+    hipError_t e;
+
+    if (event == NULL) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    e = hipEventQuery(mc_rocm_event_of(event)->hip_event);
+    if (e == hipSuccess) {
+        return XCCL_OK;
+    }
+    if (e == hipErrorNotReady) {
+        return XCCL_INPROGRESS;
+    }
+    return XCCL_ERR_NO_MESSAGE;
+}
+
+static xccl_status_t mc_rocm_event_wait(xccl_mc_event_t *event)
+{
+    if (event == NULL) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    MC_HIP(hipEventSynchronize(mc_rocm_event_of(event)->hip_event));
+    return XCCL_OK;
+}
+
+static xccl_status_t mc_rocm_event_free(xccl_mc_event_t *event)
+{
+    if (event == NULL) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    atomic_store(&mc_rocm_event_of(event)->is_free, 1);
+    return XCCL_OK;
+}
+
+/* cuda_mem_component.c:139-162: block the USER's stream until the host calls
+ * finish_stream_activity.  A gate kernel on the component stream polls a
+ * host-mapped word; the user stream waits on an event recorded behind it. */
+static xccl_status_t
+mc_rocm_start_stream_activity(xccl_stream_t *stream,
+                              xccl_mem_component_stream_request_t **req)
+{
+    mc_rocm_device_t         *d;
+    mc_rocm_stream_request_t *r = NULL;
+    hipStream_t               user;
+    xccl_status_t             st;
+    int                       i, expect;
+
+    st = mc_rocm_user_stream(stream, &user);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    st = mc_rocm_device(&d);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS && r == NULL; i++) {
+        expect = MC_SLOT_FREE;
+        if (atomic_compare_exchange_strong(&d->requests[i].is_free, &expect,
+                                           MC_SLOT_BUSY)) {
+            r = &d->requests[i];
+        } else if (expect == MC_SLOT_DRAINING &&
+                   hipEventQuery(d->requests[i].hip_event) == hipSuccess &&
+                   atomic_compare_exchange_strong(&d->requests[i].is_free,
+                                                  &expect, MC_SLOT_BUSY)) {
+            r = &d->requests[i]; /* its previous gate kernel has retired */
+        }
+    }
+    if (r == NULL) {
+        return XCCL_ERR_NO_RESOURCE;
+    }
+    __atomic_store_n(r->flag, 0, __ATOMIC_RELEASE);
+    st = xccl_rocm_stream_gate(r->dev_flag, mc_gate_timeout_ns, d->stream);
+    if (st != XCCL_OK) {
+        atomic_store(&r->is_free, 1);
+        return st;
+    }
+    if (hipEventRecord(r->hip_event, d->stream) != hipSuccess ||
+        hipStreamWaitEvent(user, r->hip_event, 0) != hipSuccess) {
+        /* open the gate again: nothing may stay blocked behind a failure */
+        __atomic_store_n(r->flag, 1, __ATOMIC_RELEASE);
+        atomic_store(&r->is_free, 1);
+        return XCCL_ERR_NO_MESSAGE;
+    }
+    r->super.mem_type = UCS_MEMORY_TYPE_ROCM;
+    *req              = &r->super;
+    return XCCL_OK;
+}
+
+static xccl_status_t
+mc_rocm_finish_stream_activity(xccl_mem_component_stream_request_t *req)
+{
+    mc_rocm_stream_request_t *r;
+
+    if (req == NULL) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    r = (mc_rocm_stream_request_t *)((char *)req -
+                                     offsetof(mc_rocm_stream_request_t, super));
+    __atomic_store_n(r->flag, 1, __ATOMIC_RELEASE);
+    /* Not reusable until its gate kernel has seen the word and left the
+     * queue; start_stream_activity checks that when it claims the slot. */
+    atomic_store(&r->is_free, MC_SLOT_DRAINING);
+    return XCCL_OK;
+}
+
+static xccl_status_t mc_rocm_get_stream(void **hip_stream)
+{
+    mc_rocm_device_t *d;
+    xccl_status_t     st = mc_rocm_device(&d);
+
+    if (st != XCCL_OK) {
+        return st;
+    }
+    *hip_stream = (void *)d->stream;
+    return XCCL_OK;
+}
+
+/* Releases the current device's resources (the reference component owns one
+ * device's worth, cuda_mem_component.c:251-265). */
+static void mc_rocm_close(void)
+{
+    mc_rocm_device_t *d;
+    int               dev = 0, i;
+
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MC_MAX_DEVICES) {
+        (void)hipGetLastError();
+        return;
+    }
+    d = &mc_devices[dev];
+    pthread_mutex_lock(&mc_init_lock);
+    if (atomic_load(&d->ready) == 1) {
+        (void)hipStreamSynchronize(d->stream);
+        xccl_rocm_graph_cache_destroy();
+        for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
+            (void)hipEventDestroy(d->events[i].hip_event);
+        }
+        for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS; i++) {
+            (void)hipEventDestroy(d->requests[i].hip_event);
+        }
+        (void)hipHostFree(d->gate_words);
+        (void)hipStreamDestroy(d->stream);
+        memset(d, 0, sizeof(*d));
+    }
+    pthread_mutex_unlock(&mc_init_lock);
+}
+
+xccl_rocm_mem_component_t xccl_rocm_mem_component = {
+    .super = {
+        .open                   = mc_rocm_open,
+        .mem_alloc              = mc_rocm_mem_alloc,
+        .mem_free               = mc_rocm_mem_free,
+        .mem_type               = mc_rocm_mem_type,
+        .reduce                 = mc_rocm_reduce,
+        .reduce_multi           = mc_rocm_reduce_multi,
+        .memcpy_async           = mc_rocm_memcpy_async,
+        .event_record           = mc_rocm_event_record,
+        .event_query            = mc_rocm_event_query,
+        .event_free             = mc_rocm_event_free,
+        .start_stream_activity  = mc_rocm_start_stream_activity,
+        .finish_stream_activity = mc_rocm_finish_stream_activity,
+        .close                  = mc_rocm_close,
+    },
+    .ext_version     = XCCL_ROCM_MC_EXT_VERSION,
+    .reduce_nb       = mc_rocm_reduce_nb,
+    .reduce_multi_nb = mc_rocm_reduce_multi_nb,
+    .event_wait      = mc_rocm_event_wait,
+    .get_stream      = mc_rocm_get_stream,
+};
+
+/* The reference loader asks every component file for this one name
+ * (src/utils/mem_component.c:30). */
+extern xccl_rocm_mem_component_t xccl_cuda_mem_component
+    __attribute__((alias("xccl_rocm_mem_component")));

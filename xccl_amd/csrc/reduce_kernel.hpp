@@ -1,0 +1,297 @@
+// reduce_kernel.hpp -- the one gfx950 kernel template behind reduce and
+// reduce_multi, and the per-(type, op) table entries built from it.
+//
+// What it computes (reference src/utils/mem_component.c:133-139 for the fold,
+// src/utils/reduce.h:14-23 for the operators):
+//     acc = OP(sbuf1[i], sbuf2{0}[i]);  acc = OP(sbuf2{j}[i], acc), j = 1..n-1
+//     rbuf[i] = acc
+// The reference's CUDA kernel (xccl_cuda_reduce_multi.cu:17-40) keeps acc in
+// global memory and reads 2/4/8 bytes per lane; here every lane moves 16 bytes
+// per source with one global_load_dwordx4, all sources of a tile are in flight
+// before the first fold, and acc never leaves registers.
+//
+// Layout of one call, in elements of T:
+//     [0, head)                 peeled so that the vector body starts on a
+//                               16-byte boundary of the buffer chosen by the
+//                               host (fewer than 16/sizeof(T) elements)
+//     [head, head + nvec*VE)    nvec 16-byte vectors, VE = 16/sizeof(T)
+//     [.., .. + tail)           fewer than VE elements
+// Head and tail are folded element-wise by the first lanes of the last block.
+// Vector accesses are emitted as dwordx4 whatever the address is (the device
+// runs in unaligned access mode), so a source whose alignment differs from
+// the peeled one costs extra cache-line touches, never correctness.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace xccl_rocm {
+
+constexpr int kBlock = 256;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_u __attribute__((aligned(1)));
+
+struct ReduceArgs {
+    const char *s1;     // sbuf1
+    const char *s2;     // sbuf2 (vector 0)
+    char       *dst;    // rbuf / target
+    size_t      stride; // bytes between vectors of sbuf2
+    size_t      head;   // elements before the vector body
+    size_t      nvec;   // 16-byte vectors in the body
+    size_t      tail;   // elements after the vector body
+    uint32_t    n2;     // vectors in sbuf2 (>= 1)
+};
+
+// ---- operators: reduce.h:14-23, first macro argument = a ------------------
+// Integer kernels run on unsigned types wherever the result bits do not
+// depend on signedness (SUM, PROD, logical, bitwise), which also makes
+// wrap-around defined; MIN/MAX are instantiated for both signednesses.
+struct OpMax  { template <class T> static __device__ __forceinline__ T f(T a, T b) { return a > b ? a : b; } };
+struct OpMin  { template <class T> static __device__ __forceinline__ T f(T a, T b) { return a < b ? a : b; } };
+struct OpSum  { template <class T> static __device__ __forceinline__ T f(T a, T b) { return (T)(a + b); } };
+struct OpProd { template <class T> static __device__ __forceinline__ T f(T a, T b) { return (T)(a * b); } };
+struct OpLand { template <class T> static __device__ __forceinline__ T f(T a, T b) { return (T)(a && b); } };
+struct OpLor  { template <class T> static __device__ __forceinline__ T f(T a, T b) { return (T)(a || b); } };
+struct OpLxor { template <class T> static __device__ __forceinline__ T f(T a, T b) { return (T)((!a) != (!b)); } };
+struct OpBand { template <class T> static __device__ __forceinline__ T f(T a, T b) { return (T)(a & b); } };
+struct OpBor  { template <class T> static __device__ __forceinline__ T f(T a, T b) { return (T)(a | b); } };
+struct OpBxor { template <class T> static __device__ __forceinline__ T f(T a, T b) { return (T)(a ^ b); } };
+
+// uint16 * uint16 promotes to (signed) int and can overflow it; multiply in
+// 32-bit unsigned and truncate, which is what the promoted product's low bits
+// are.
+template <> __device__ __forceinline__ uint16_t OpProd::f<uint16_t>(uint16_t a, uint16_t b)
+{
+    return (uint16_t)((uint32_t)a * (uint32_t)b);
+}
+
+template <typename T> struct Vec {
+    static constexpr int n = 16 / sizeof(T);
+    typedef T type __attribute__((ext_vector_type(16 / sizeof(T))));
+};
+
+template <typename T, class Op>
+__device__ __forceinline__ u32x4 vfold(u32x4 a, u32x4 b)
+{
+    typedef typename Vec<T>::type V;
+    V x = __builtin_bit_cast(V, a);
+    V y = __builtin_bit_cast(V, b);
+    V r;
+#pragma unroll
+    for (int k = 0; k < Vec<T>::n; ++k) {
+        r[k] = Op::template f<T>(x[k], y[k]);
+    }
+    return __builtin_bit_cast(u32x4, r);
+}
+
+// Bitwise operators do not care where element boundaries are.
+template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBand>(u32x4 a, u32x4 b) { return a & b; }
+template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBor>(u32x4 a, u32x4 b)  { return a | b; }
+template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBxor>(u32x4 a, u32x4 b) { return a ^ b; }
+
+template <bool NT>
+__device__ __forceinline__ u32x4 vload(const char *p)
+{
+    if (NT) {
+        return __builtin_nontemporal_load((const u32x4_u *)p);
+    }
+    return *(const u32x4_u *)p;
+}
+
+template <bool NT>
+__device__ __forceinline__ void vstore(char *p, u32x4 v)
+{
+    if (NT) {
+        __builtin_nontemporal_store(v, (u32x4_u *)p);
+    } else {
+        *(u32x4_u *)p = v;
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ T eload(const char *p)
+{
+    T v;
+    __builtin_memcpy(&v, p, sizeof(T));
+    return v;
+}
+
+// One element, all sources, in fold order.
+template <typename T, class Op>
+__device__ __forceinline__ void fold_element(const ReduceArgs &a, size_t e)
+{
+    const size_t off = e * sizeof(T);
+    T acc = Op::template f<T>(eload<T>(a.s1 + off), eload<T>(a.s2 + off));
+    for (uint32_t j = 1; j < a.n2; ++j) {
+        acc = Op::template f<T>(eload<T>(a.s2 + (size_t)j * a.stride + off), acc);
+    }
+    __builtin_memcpy(a.dst + off, &acc, sizeof(T));
+}
+
+// One tile = UNROLL x kBlock vectors; lane t of the block owns vectors
+// v0 + u*kBlock + t.  NSRC > 0: exactly NSRC sources, all NSRC*UNROLL loads
+// issued before the first fold.  NSRC == 0: any number of sources, loaded four
+// at a time.  GUARD: the tile may run past nvec.
+template <typename T, class Op, int NSRC, int UNROLL, bool NT, bool GUARD>
+__device__ __forceinline__ void fold_tile(const ReduceArgs &a, size_t v0)
+{
+    const size_t body = a.head * sizeof(T);
+    size_t       off[UNROLL];
+    bool         live[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const size_t v = v0 + (size_t)u * kBlock + threadIdx.x;
+        live[u]        = !GUARD || v < a.nvec;
+        off[u]         = body + v * 16;
+    }
+
+    if constexpr (NSRC > 0) {
+        constexpr int N = NSRC;
+        u32x4         r[UNROLL][N];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (live[u]) {
+                r[u][0] = vload<NT>(a.s1 + off[u]);
+#pragma unroll
+                for (int j = 1; j < N; ++j) {
+                    r[u][j] = vload<NT>(a.s2 + (size_t)(j - 1) * a.stride + off[u]);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (live[u]) {
+                u32x4 acc = vfold<T, Op>(r[u][0], r[u][1]);
+#pragma unroll
+                for (int j = 2; j < N; ++j) {
+                    acc = vfold<T, Op>(r[u][j], acc);
+                }
+                vstore<NT>(a.dst + off[u], acc);
+            }
+        }
+    } else {
+        u32x4 acc[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (live[u]) {
+                u32x4 x = vload<NT>(a.s1 + off[u]);
+                u32x4 y = vload<NT>(a.s2 + off[u]);
+                acc[u]  = vfold<T, Op>(x, y);
+            }
+        }
+        uint32_t j = 1;
+        for (; j + 4 <= a.n2; j += 4) {
+            const char *p = a.s2 + (size_t)j * a.stride;
+            u32x4       r[UNROLL][4];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (live[u]) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        r[u][k] = vload<NT>(p + (size_t)k * a.stride + off[u]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (live[u]) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        acc[u] = vfold<T, Op>(r[u][k], acc[u]);
+                    }
+                }
+            }
+        }
+        for (; j < a.n2; ++j) {
+            const char *p = a.s2 + (size_t)j * a.stride;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (live[u]) {
+                    acc[u] = vfold<T, Op>(vload<NT>(p + off[u]), acc[u]);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (live[u]) {
+                vstore<NT>(a.dst + off[u], acc[u]);
+            }
+        }
+    }
+}
+
+template <typename T, class Op, int NSRC, int UNROLL, bool NT>
+__global__ void __launch_bounds__(kBlock) reduce_multi_kernel(const ReduceArgs a)
+{
+    constexpr size_t tile = (size_t)kBlock * UNROLL;
+    const size_t     step = (size_t)gridDim.x * tile;
+    for (size_t v0 = (size_t)blockIdx.x * tile; v0 < a.nvec; v0 += step) {
+        if (v0 + tile <= a.nvec) {
+            fold_tile<T, Op, NSRC, UNROLL, NT, false>(a, v0);
+        } else {
+            fold_tile<T, Op, NSRC, UNROLL, NT, true>(a, v0);
+        }
+    }
+    if (blockIdx.x == gridDim.x - 1) {
+        const size_t t = threadIdx.x;
+        if (t < a.head) {
+            fold_element<T, Op>(a, t);
+        } else if (t - a.head < a.tail) {
+            fold_element<T, Op>(a, a.head + a.nvec * Vec<T>::n + (t - a.head));
+        }
+    }
+}
+
+// ---- table of instantiations ---------------------------------------------
+// Source-count variants: exact counts for the radices the k-nomial and
+// scatter-reduce steps use (2, 3, 4, 8, 16 sources), and the any-count kernel.
+enum { NV_ANY = 0, NV_2, NV_3, NV_4, NV_8, NV_16, NV_COUNT };
+
+constexpr int nsrc_of(int nv) { return nv == NV_2 ? 2 : nv == NV_3 ? 3 : nv == NV_4 ? 4 : nv == NV_8 ? 8 : nv == NV_16 ? 16 : 0; }
+// vectors per lane per tile
+constexpr int unroll_of(int nv) { return nv == NV_2 ? 4 : nv == NV_3 ? 4 : nv == NV_4 ? 2 : nv == NV_8 ? 2 : nv == NV_16 ? 1 : 2; }
+
+struct KernelEntry {
+    const void *fn[2][NV_COUNT]; // [nontemporal][variant]
+    int         elem_size;       // sizeof(T) the kernel folds in
+};
+
+template <typename T, class Op, bool NT, int NV>
+constexpr const void *kernel_ptr()
+{
+    return (const void *)&reduce_multi_kernel<T, Op, nsrc_of(NV), unroll_of(NV), NT>;
+}
+
+template <typename T, class Op>
+KernelEntry make_entry()
+{
+    KernelEntry e;
+    e.fn[0][NV_ANY] = kernel_ptr<T, Op, false, NV_ANY>();
+    e.fn[0][NV_2]   = kernel_ptr<T, Op, false, NV_2>();
+    e.fn[0][NV_3]   = kernel_ptr<T, Op, false, NV_3>();
+    e.fn[0][NV_4]   = kernel_ptr<T, Op, false, NV_4>();
+    e.fn[0][NV_8]   = kernel_ptr<T, Op, false, NV_8>();
+    e.fn[0][NV_16]  = kernel_ptr<T, Op, false, NV_16>();
+    e.fn[1][NV_ANY] = kernel_ptr<T, Op, true, NV_ANY>();
+    e.fn[1][NV_2]   = kernel_ptr<T, Op, true, NV_2>();
+    e.fn[1][NV_3]   = kernel_ptr<T, Op, true, NV_3>();
+    e.fn[1][NV_4]   = kernel_ptr<T, Op, true, NV_4>();
+    e.fn[1][NV_8]   = kernel_ptr<T, Op, true, NV_8>();
+    e.fn[1][NV_16]  = kernel_ptr<T, Op, true, NV_16>();
+    e.elem_size     = (int)sizeof(T);
+    return e;
+}
+
+// Operator slots of a per-type table.
+enum { K_MAX = 0, K_MIN, K_SUM, K_PROD, K_LAND, K_LOR, K_LXOR, K_BAND, K_BOR, K_BXOR, K_COUNT };
+
+// One translation unit per element width keeps the build parallel.  Each
+// returns NULL for a slot it does not implement.
+const KernelEntry *lookup_w8(int kop, bool is_signed);
+const KernelEntry *lookup_w16(int kop, bool is_signed);
+const KernelEntry *lookup_w32(int kop, bool is_signed);
+const KernelEntry *lookup_w64(int kop, bool is_signed);
+const KernelEntry *lookup_fp(int kop, int bytes); // bytes = 2, 4, 8; K_MAX..K_PROD
+
+} // namespace xccl_rocm

@@ -1,0 +1,445 @@
+// reduce_launch.hip -- host side of the kernel ABI declared in
+// include/xccl_rocm_kernels.h: (dtype, op) -> kernel lookup, launch planning,
+// plain launch, the cached single-node hipGraph launch, and the stream gate.
+#include "reduce_kernel.hpp"
+#include "xccl_rocm_kernels.h"
+
+#include <atomic>
+#include <mutex>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+namespace xccl_rocm {
+namespace {
+
+constexpr int kMaxDevices       = 64;
+constexpr int kDefaultBlocksPerCu = 8; // 8 x 256 lanes = every wave slot of a CU
+
+std::atomic<int> g_blocks_per_cu{-1}; // -1: not read from the environment yet
+std::atomic<int> g_nontemporal{-1};
+std::atomic<int> g_cu_count[kMaxDevices];
+
+void read_env_once()
+{
+    if (g_blocks_per_cu.load(std::memory_order_acquire) >= 0) {
+        return;
+    }
+    const char *nt  = getenv("XCCL_MC_ROCM_NONTEMPORAL");
+    const char *bpc = getenv("XCCL_MC_ROCM_BLOCKS_PER_CU");
+    int         v   = bpc ? atoi(bpc) : 0;
+    g_nontemporal.store((nt && atoi(nt) != 0) ? 1 : 0, std::memory_order_release);
+    g_blocks_per_cu.store(v > 0 ? v : kDefaultBlocksPerCu, std::memory_order_release);
+}
+
+// Compute units of the current device (cached per device ordinal).
+xccl_status_t cu_count(int *cus)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        return XCCL_ERR_NO_MESSAGE;
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        return XCCL_ERR_NO_RESOURCE;
+    }
+    int n = g_cu_count[dev].load(std::memory_order_acquire);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            return XCCL_ERR_NO_MESSAGE;
+        }
+        g_cu_count[dev].store(n, std::memory_order_release);
+    }
+    *cus = n;
+    return XCCL_OK;
+}
+
+int kop_of(xccl_op_t op)
+{
+    switch (op) {
+    case XCCL_OP_MAX:  return K_MAX;
+    case XCCL_OP_MIN:  return K_MIN;
+    case XCCL_OP_SUM:  return K_SUM;
+    case XCCL_OP_PROD: return K_PROD;
+    case XCCL_OP_LAND: return K_LAND;
+    case XCCL_OP_LOR:  return K_LOR;
+    case XCCL_OP_LXOR: return K_LXOR;
+    case XCCL_OP_BAND: return K_BAND;
+    case XCCL_OP_BOR:  return K_BOR;
+    case XCCL_OP_BXOR: return K_BXOR;
+    default:           return -1; // AND/OR/XOR/MAXLOC/MINLOC: no kernel
+    }
+}
+
+// The kernel family for (dtype, op), or NULL.  Coverage follows the
+// reference kernels' switch (xccl_cuda_reduce_multi.cu:118-138) widened to
+// 8-bit, unsigned and binary16 element types.
+const KernelEntry *lookup(xccl_dt_t dt, xccl_op_t op)
+{
+    const int kop = kop_of(op);
+    if (kop < 0) {
+        return nullptr;
+    }
+    bool is_signed = false;
+    int  bytes     = 0;
+    switch (dt) {
+    case XCCL_DT_INT8:   is_signed = true; bytes = 1; break;
+    case XCCL_DT_INT16:  is_signed = true; bytes = 2; break;
+    case XCCL_DT_INT32:  is_signed = true; bytes = 4; break;
+    case XCCL_DT_INT64:  is_signed = true; bytes = 8; break;
+    case XCCL_DT_UINT8:  bytes = 1; break;
+    case XCCL_DT_UINT16: bytes = 2; break;
+    case XCCL_DT_UINT32: bytes = 4; break;
+    case XCCL_DT_UINT64: bytes = 8; break;
+    case XCCL_DT_FLOAT16: return lookup_fp(kop, 2);
+    case XCCL_DT_FLOAT32: return lookup_fp(kop, 4);
+    case XCCL_DT_FLOAT64: return lookup_fp(kop, 8);
+    default:             return nullptr; // 128-bit integers, unknown
+    }
+    if (kop >= K_BAND) {
+        return lookup_w8(kop, false);
+    }
+    switch (bytes) {
+    case 1:  return lookup_w8(kop, is_signed);
+    case 2:  return lookup_w16(kop, is_signed);
+    case 4:  return lookup_w32(kop, is_signed);
+    default: return lookup_w64(kop, is_signed);
+    }
+}
+
+struct Plan {
+    const void *fn;
+    unsigned    grid;
+    ReduceArgs  args;
+};
+
+bool same_plan(const Plan &a, const Plan &b)
+{
+    return a.fn == b.fn && a.grid == b.grid && a.args.s1 == b.args.s1 && a.args.s2 == b.args.s2 &&
+           a.args.dst == b.args.dst && a.args.stride == b.args.stride && a.args.head == b.args.head &&
+           a.args.nvec == b.args.nvec && a.args.tail == b.args.tail && a.args.n2 == b.args.n2;
+}
+
+// Bytes to peel so that as many of the buffers as possible start their
+// vector body on a 16-byte boundary; ties go to the destination.
+size_t pick_head_bytes(const void *s1, const void *s2, const void *dst, size_t stride, uint32_t n2, size_t esize)
+{
+    unsigned votes[16] = {0};
+    votes[(uintptr_t)s1 & 15]++;
+    const uint32_t look = n2 < 32 ? n2 : 32;
+    for (uint32_t j = 0; j < look; ++j) {
+        votes[((uintptr_t)s2 + (size_t)j * stride) & 15]++;
+    }
+    const unsigned dm = (unsigned)((uintptr_t)dst & 15);
+    votes[dm]++;
+    unsigned best = 16, best_votes = 0;
+    for (unsigned m = 0; m < 16; ++m) {
+        if (m % esize != 0 || votes[m] == 0) {
+            continue; // cannot be reached by peeling whole elements
+        }
+        if (votes[m] > best_votes || (votes[m] == best_votes && m == dm)) {
+            best       = m;
+            best_votes = votes[m];
+        }
+    }
+    return best == 16 ? 0 : (16 - best) % 16;
+}
+
+xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size, size_t stride, xccl_dt_t dt,
+                        xccl_op_t op, Plan *plan)
+{
+    const KernelEntry *e = lookup(dt, op);
+    if (e == nullptr) {
+        return XCCL_ERR_UNSUPPORTED;
+    }
+    if (s1 == nullptr || s2 == nullptr || dst == nullptr) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    if (count > 0xffffffffu) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    read_env_once();
+    int cus = 0;
+    xccl_status_t st = cu_count(&cus);
+    if (st != XCCL_OK) {
+        return st;
+    }
+
+    const size_t   esize = (size_t)e->elem_size;
+    const size_t   elems = size * (xccl_dt_size(dt) / esize); // bitwise ops fold bytes
+    const size_t   ve    = 16 / esize;
+    const uint32_t n2    = count == 0 ? 1u : (uint32_t)count;
+    const uint32_t nsrc  = n2 + 1;
+    const int      nv    = nsrc == 2 ? NV_2 : nsrc == 3 ? NV_3 : nsrc == 4 ? NV_4 : nsrc == 8 ? NV_8 : nsrc == 16 ? NV_16 : NV_ANY;
+
+    size_t head = pick_head_bytes(s1, s2, dst, stride, n2, esize) / esize;
+    if (head > elems) {
+        head = elems;
+    }
+    ReduceArgs &a = plan->args;
+    a.s1     = (const char *)s1;
+    a.s2     = (const char *)s2;
+    a.dst    = (char *)dst;
+    a.stride = stride;
+    a.head   = head;
+    a.nvec   = (elems - head) / ve;
+    a.tail   = (elems - head) % ve;
+    a.n2     = n2;
+
+    const size_t tile  = (size_t)kBlock * unroll_of(nv);
+    const size_t tiles = (a.nvec + tile - 1) / tile;
+    const size_t cap   = (size_t)cus * (size_t)g_blocks_per_cu.load(std::memory_order_relaxed);
+    size_t       grid  = tiles < cap ? tiles : cap;
+    if (grid == 0) {
+        grid = 1; // head/tail only
+    }
+    plan->grid = (unsigned)grid;
+    plan->fn   = e->fn[g_nontemporal.load(std::memory_order_relaxed) ? 1 : 0][nv];
+    return XCCL_OK;
+}
+
+// ---- single-kernel-node graph cache ---------------------------------------
+constexpr int kGraphSlots = 8;
+
+struct GraphSlot {
+    bool            live = false;
+    Plan            plan;
+    hipGraph_t      graph = nullptr;
+    hipGraphNode_t  node  = nullptr;
+    hipGraphExec_t  exec  = nullptr;
+    hipEvent_t      done  = nullptr; // recorded after the last launch
+    uint64_t        stamp = 0;
+};
+
+struct GraphCache {
+    std::mutex lock;
+    GraphSlot  slot[kGraphSlots];
+    uint64_t   clock = 0;
+};
+
+GraphCache g_graphs[kMaxDevices];
+
+void fill_node_params(hipKernelNodeParams *p, Plan *plan, void **argv)
+{
+    argv[0] = &plan->args;
+    memset(p, 0, sizeof(*p));
+    p->func           = const_cast<void *>(plan->fn);
+    p->gridDim        = dim3(plan->grid, 1, 1);
+    p->blockDim       = dim3(kBlock, 1, 1);
+    p->sharedMemBytes = 0;
+    p->kernelParams   = argv;
+    p->extra          = nullptr;
+}
+
+void destroy_slot(GraphSlot &s)
+{
+    if (s.exec) {
+        (void)hipGraphExecDestroy(s.exec);
+    }
+    if (s.graph) {
+        (void)hipGraphDestroy(s.graph);
+    }
+    if (s.done) {
+        (void)hipEventDestroy(s.done);
+    }
+    s = GraphSlot();
+}
+
+#define HIP_OR_FAIL(call)                                                                          \
+    do {                                                                                           \
+        hipError_t e_ = (call);                                                                    \
+        if (e_ != hipSuccess) {                                                                    \
+            fprintf(stderr, "xccl mc_rocm: %s failed: %s\n", #call, hipGetErrorString(e_));        \
+            return XCCL_ERR_NO_MESSAGE;                                                            \
+        }                                                                                          \
+    } while (0)
+
+xccl_status_t graph_launch(Plan &plan, hipStream_t stream)
+{
+    int dev = 0;
+    HIP_OR_FAIL(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) {
+        return XCCL_ERR_NO_RESOURCE;
+    }
+    GraphCache                 &gc = g_graphs[dev];
+    std::lock_guard<std::mutex> guard(gc.lock);
+
+    GraphSlot *hit = nullptr, *victim = nullptr;
+    for (GraphSlot &s : gc.slot) {
+        if (s.live && same_plan(s.plan, plan)) {
+            hit = &s;
+            break;
+        }
+    }
+    if (hit == nullptr) {
+        for (GraphSlot &s : gc.slot) { // a free slot, else the least recently used
+            if (!s.live) {
+                victim = &s;
+                break;
+            }
+            if (victim == nullptr || s.stamp < victim->stamp) {
+                victim = &s;
+            }
+        }
+    }
+
+    if (hit == nullptr) {
+        hipKernelNodeParams np;
+        void               *argv[1];
+        if (!victim->live) {
+            victim->plan = plan;
+            fill_node_params(&np, &victim->plan, argv);
+            HIP_OR_FAIL(hipGraphCreate(&victim->graph, 0));
+            if (hipGraphAddKernelNode(&victim->node, victim->graph, nullptr, 0, &np) != hipSuccess ||
+                hipGraphInstantiate(&victim->exec, victim->graph, nullptr, nullptr, 0) != hipSuccess ||
+                hipEventCreateWithFlags(&victim->done, hipEventDisableTiming) != hipSuccess) {
+                destroy_slot(*victim);
+                (void)hipGetLastError();
+                return XCCL_ERR_NO_MESSAGE;
+            }
+            victim->live = true;
+        } else {
+            // The executable graph may still be running its previous launch
+            // on another stream; patch it only once that launch has finished.
+            HIP_OR_FAIL(hipEventSynchronize(victim->done));
+            victim->plan = plan;
+            fill_node_params(&np, &victim->plan, argv);
+            if (hipGraphExecKernelNodeSetParams(victim->exec, victim->node, &np) != hipSuccess) {
+                destroy_slot(*victim);
+                (void)hipGetLastError();
+                return XCCL_ERR_NO_MESSAGE;
+            }
+        }
+        hit = victim;
+    }
+    hit->stamp = ++gc.clock;
+    HIP_OR_FAIL(hipGraphLaunch(hit->exec, stream));
+    HIP_OR_FAIL(hipEventRecord(hit->done, stream));
+    return XCCL_OK;
+}
+
+// Polls *flag (host-mapped) from one lane; see xccl_rocm_stream_gate.
+__global__ void stream_gate_kernel(int *flag, uint64_t max_ticks)
+{
+    const uint64_t t0 = wall_clock64();
+    while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == 0) {
+        if (wall_clock64() - t0 > max_ticks) {
+            __hip_atomic_store(flag, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(16);
+    }
+}
+
+} // namespace
+} // namespace xccl_rocm
+
+using namespace xccl_rocm;
+
+extern "C" {
+
+xccl_status_t xccl_rocm_reduce_supported(xccl_dt_t dtype, xccl_op_t op)
+{
+    return lookup(dtype, op) ? XCCL_OK : XCCL_ERR_UNSUPPORTED;
+}
+
+xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
+                                          size_t stride, xccl_dt_t dtype, xccl_op_t op, void *hip_stream)
+{
+    if (lookup(dtype, op) == nullptr) {
+        return XCCL_ERR_UNSUPPORTED;
+    }
+    if (size == 0) {
+        return XCCL_OK;
+    }
+    Plan          plan;
+    xccl_status_t st = make_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    void *argv[1] = {&plan.args};
+    HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, 0, (hipStream_t)hip_stream));
+    return XCCL_OK;
+}
+
+xccl_status_t xccl_rocm_reduce_impl(void *sbuf1, void *sbuf2, void *target, size_t count, xccl_dt_t dtype,
+                                    xccl_op_t op, void *hip_stream)
+{
+    return xccl_rocm_reduce_multi_impl(sbuf1, sbuf2, target, 1, count, 0, dtype, op, hip_stream);
+}
+
+xccl_status_t xccl_rocm_reduce_multi_graph(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
+                                           size_t stride, xccl_dt_t dtype, xccl_op_t op, void *hip_stream)
+{
+    if (lookup(dtype, op) == nullptr) {
+        return XCCL_ERR_UNSUPPORTED;
+    }
+    if (size == 0) {
+        return XCCL_OK;
+    }
+    Plan          plan;
+    xccl_status_t st = make_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    return graph_launch(plan, (hipStream_t)hip_stream);
+}
+
+void xccl_rocm_graph_cache_destroy(void)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return;
+    }
+    GraphCache                 &gc = g_graphs[dev];
+    std::lock_guard<std::mutex> guard(gc.lock);
+    for (GraphSlot &s : gc.slot) {
+        if (s.live) {
+            (void)hipEventSynchronize(s.done);
+        }
+        destroy_slot(s);
+    }
+}
+
+void xccl_rocm_set_launch_shape(int blocks_per_cu, int nontemporal)
+{
+    read_env_once();
+    g_blocks_per_cu.store(blocks_per_cu > 0 ? blocks_per_cu : kDefaultBlocksPerCu, std::memory_order_release);
+    g_nontemporal.store(nontemporal ? 1 : 0, std::memory_order_release);
+}
+
+xccl_status_t xccl_rocm_reduce_multi_plan(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
+                                          size_t stride, xccl_dt_t dtype, xccl_op_t op, unsigned *grid,
+                                          unsigned *block, char *name, size_t name_len)
+{
+    Plan          plan;
+    xccl_status_t st = make_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    if (grid) {
+        *grid = plan.grid;
+    }
+    if (block) {
+        *block = kBlock;
+    }
+    if (name && name_len > 0) {
+        const char *n = hipKernelNameRefByPtr(plan.fn, nullptr);
+        snprintf(name, name_len, "%s", n ? n : "");
+    }
+    return XCCL_OK;
+}
+
+xccl_status_t xccl_rocm_stream_gate(int *dev_flag, uint64_t max_ns, void *hip_stream)
+{
+    if (dev_flag == nullptr) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    // wall_clock64() counts at 100 MHz on gfx950.
+    const uint64_t ticks = max_ns / 10 + 1;
+    hipLaunchKernelGGL(stream_gate_kernel, dim3(1), dim3(1), 0, (hipStream_t)hip_stream, dev_flag, ticks);
+    HIP_OR_FAIL(hipGetLastError());
+    return XCCL_OK;
+}
+
+} // extern "C"

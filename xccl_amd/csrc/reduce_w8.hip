@@ -1,0 +1,34 @@
+// reduce_w8.hip -- 8-bit integer instantiations of the reduction kernel.
+// SUM, PROD, the logical and the bitwise operators give the same bits for
+// int8_t and uint8_t, so they are built once, on the unsigned type;
+// MAX and MIN are built for both.
+// The bitwise operators of every width run here, on bytes.
+#include "reduce_kernel.hpp"
+
+namespace xccl_rocm {
+
+const KernelEntry *lookup_w8(int kop, bool is_signed)
+{
+    typedef uint8_t U;
+    typedef int8_t  S;
+    static const KernelEntry common[K_COUNT] = {
+        make_entry<U, OpMax>(),  make_entry<U, OpMin>(),  make_entry<U, OpSum>(),
+        make_entry<U, OpProd>(), make_entry<U, OpLand>(), make_entry<U, OpLor>(),
+        make_entry<U, OpLxor>(),
+        make_entry<U, OpBand>(), make_entry<U, OpBor>(),  make_entry<U, OpBxor>(),
+    };
+    static const KernelEntry smax = make_entry<S, OpMax>();
+    static const KernelEntry smin = make_entry<S, OpMin>();
+    if (kop < 0 || kop >= K_COUNT) {
+        return nullptr;
+    }
+    if (is_signed && kop == K_MAX) {
+        return &smax;
+    }
+    if (is_signed && kop == K_MIN) {
+        return &smin;
+    }
+    return &common[kop];
+}
+
+} // namespace xccl_rocm

@@ -1,0 +1,305 @@
+"""ctypes mirror of the mem-component boundary (include/xccl_rocm_mem_component.h,
+include/xccl_rocm_kernels.h).
+
+Function names, argument order and status codes are those of the reference
+dispatcher (src/utils/mem_component.h:52-95); every function returns the
+``xccl_status_t`` as ``Status`` and raises nothing for an XCCL error, so tests
+can assert on codes the way the reference's callers would.  Loading fails
+loudly when the libraries are not built -- there is no Python or CPU stand-in
+for the arithmetic.
+"""
+import ctypes
+import os
+
+from .build import LIB_DIR, built
+from .types import MemType, Status, StreamType
+
+_c = ctypes
+_vp, _sz, _int = _c.c_void_p, _c.c_size_t, _c.c_int
+
+
+class XcclStream(_c.Structure):
+    """xccl_stream_t: ``stream`` points AT a hipStream_t."""
+    _fields_ = [("type", _int), ("stream", _vp)]
+
+
+class McBuf(_c.Structure):
+    _fields_ = [("buf", _vp), ("size", _sz), ("used", _int)]
+
+
+_ST = _int  # xccl_status_t
+
+
+class MemComponentVtable(_c.Structure):
+    """xccl_mem_component_t (reference src/utils/mem_component.h:28-49)."""
+    _fields_ = [
+        ("open", _c.CFUNCTYPE(_ST)),
+        ("mem_alloc", _c.CFUNCTYPE(_ST, _c.POINTER(_vp), _sz)),
+        ("mem_free", _c.CFUNCTYPE(_ST, _vp)),
+        ("mem_type", _c.CFUNCTYPE(_ST, _vp, _c.POINTER(_int))),
+        ("reduce", _c.CFUNCTYPE(_ST, _vp, _vp, _vp, _sz, _int, _int)),
+        ("reduce_multi", _c.CFUNCTYPE(_ST, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int)),
+        ("memcpy_async", _c.CFUNCTYPE(_ST, _vp, _vp, _sz, _c.POINTER(XcclStream))),
+        ("event_record", _c.CFUNCTYPE(_ST, _c.POINTER(XcclStream), _c.POINTER(_vp))),
+        ("event_query", _c.CFUNCTYPE(_ST, _vp)),
+        ("event_free", _c.CFUNCTYPE(_ST, _vp)),
+        ("start_stream_activity", _c.CFUNCTYPE(_ST, _c.POINTER(XcclStream), _c.POINTER(_vp))),
+        ("finish_stream_activity", _c.CFUNCTYPE(_ST, _vp)),
+        ("close", _c.CFUNCTYPE(None)),
+        ("dlhandle", _vp),
+        ("cache", McBuf),
+    ]
+
+
+class RocmMemComponent(_c.Structure):
+    """xccl_rocm_mem_component_t: the vtable plus the stream-ordered extension."""
+    _fields_ = [
+        ("super", MemComponentVtable),
+        ("ext_version", _c.c_uint32),
+        ("reduce_nb", _c.CFUNCTYPE(_ST, _vp, _vp, _vp, _sz, _int, _int, _c.POINTER(XcclStream), _c.POINTER(_vp))),
+        ("reduce_multi_nb", _c.CFUNCTYPE(_ST, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _c.POINTER(XcclStream),
+                                         _c.POINTER(_vp))),
+        ("event_wait", _c.CFUNCTYPE(_ST, _vp)),
+        ("get_stream", _c.CFUNCTYPE(_ST, _c.POINTER(_vp))),
+    ]
+
+
+COMPONENT_SO = os.path.join(LIB_DIR, "xccl_rocm_mem_component.so")
+DISPATCH_SO = os.path.join(LIB_DIR, "libxccl_mc.so")
+BENCHKIT_SO = os.path.join(LIB_DIR, "libxccl_rocm_benchkit.so")
+
+_component_lib = None
+_dispatch_lib = None
+_datagen_lib = None
+
+
+def _need_built():
+    if not built():
+        raise RuntimeError(
+            "xccl_amd: native libraries missing under %s -- run `python -m xccl_amd.build` "
+            "(there is no CPU fallback)" % LIB_DIR)
+
+
+def component_lib():
+    """xccl_rocm_mem_component.so, loaded directly (kernel ABI + exported vtable)."""
+    global _component_lib
+    if _component_lib is None:
+        _need_built()
+        lib = _c.CDLL(COMPONENT_SO, mode=_c.RTLD_GLOBAL)
+        lib.xccl_rocm_reduce_supported.argtypes = [_int, _int]
+        lib.xccl_rocm_reduce_impl.argtypes = [_vp, _vp, _vp, _sz, _int, _int, _vp]
+        lib.xccl_rocm_reduce_multi_impl.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp]
+        lib.xccl_rocm_reduce_multi_graph.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp]
+        lib.xccl_rocm_graph_cache_destroy.argtypes = []
+        lib.xccl_rocm_graph_cache_destroy.restype = None
+        lib.xccl_rocm_set_launch_shape.argtypes = [_int, _int]
+        lib.xccl_rocm_set_launch_shape.restype = None
+        lib.xccl_rocm_reduce_multi_plan.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int,
+                                                    _c.POINTER(_c.c_uint), _c.POINTER(_c.c_uint), _c.c_char_p, _sz]
+        lib.xccl_rocm_stream_gate.argtypes = [_vp, _c.c_uint64, _vp]
+        _component_lib = lib
+    return _component_lib
+
+
+def component() -> RocmMemComponent:
+    """The exported object `xccl_rocm_mem_component`."""
+    return RocmMemComponent.in_dll(component_lib(), "xccl_rocm_mem_component")
+
+
+def dispatch_lib():
+    global _dispatch_lib
+    if _dispatch_lib is None:
+        _need_built()
+        lib = _c.CDLL(DISPATCH_SO)
+        lib.xccl_mem_component_init.argtypes = [_c.c_char_p]
+        lib.xccl_mem_component_alloc.argtypes = [_c.POINTER(_vp), _sz, _int]
+        lib.xccl_mem_component_free.argtypes = [_vp, _int]
+        lib.xccl_mem_component_type.argtypes = [_vp, _c.POINTER(_int)]
+        lib.xccl_mem_component_reduce.argtypes = [_vp, _vp, _vp, _sz, _int, _int, _int]
+        lib.xccl_mem_component_reduce_multi.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _int]
+        lib.xccl_mem_component_reduce_nb.argtypes = [_vp, _vp, _vp, _sz, _int, _int, _int, _c.POINTER(XcclStream),
+                                                     _c.POINTER(_vp)]
+        lib.xccl_mem_component_reduce_multi_nb.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _int,
+                                                           _c.POINTER(XcclStream), _c.POINTER(_vp)]
+        lib.xccl_mem_component_memcpy_async.argtypes = [_vp, _vp, _sz, _c.POINTER(XcclStream)]
+        lib.xccl_mem_component_start_acitivity.argtypes = [_c.POINTER(XcclStream), _c.POINTER(_vp)]
+        lib.xccl_mem_component_finish_acitivity.argtypes = [_vp]
+        lib.xccl_mc_event_record.argtypes = [_c.POINTER(XcclStream), _c.POINTER(_vp)]
+        lib.xccl_mc_event_query.argtypes = [_vp]
+        lib.xccl_mc_event_free.argtypes = [_vp]
+        lib.xccl_mc_event_wait.argtypes = [_vp]
+        lib.xccl_mem_component_free_cache.argtypes = []
+        lib.xccl_mem_component_free_cache.restype = None
+        lib.xccl_mem_component_finalize.argtypes = []
+        lib.xccl_mem_component_finalize.restype = None
+        lib.xccl_mem_component_get.argtypes = [_int]
+        lib.xccl_mem_component_get.restype = _c.POINTER(MemComponentVtable)
+        _dispatch_lib = lib
+    return _dispatch_lib
+
+
+def benchkit_lib():
+    global _datagen_lib
+    if _datagen_lib is None:
+        _need_built()
+        lib = _c.CDLL(BENCHKIT_SO)
+        lib.xccl_rocm_datagen_fill.argtypes = [_vp, _sz, _int, _c.c_uint64, _c.c_uint64, _int, _vp]
+        lib.xccl_rocm_bench_latency.argtypes = [_vp, _vp, _int, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
+        lib.xccl_rocm_bench_kernel_times.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp]
+        _datagen_lib = lib
+    return _datagen_lib
+
+
+def _st(code) -> Status:
+    try:
+        return Status(code)
+    except ValueError:
+        return code
+
+
+class Stream:
+    """Owns a hipStream_t and the xccl_stream_t that points at it."""
+
+    def __init__(self, hip_stream, stype=StreamType.ROCM):
+        self._handle = _vp(hip_stream)
+        self.xccl = XcclStream(int(stype), _c.cast(_c.pointer(self._handle), _vp))
+
+    @property
+    def hip_stream(self):
+        return self._handle.value
+
+    def ref(self):
+        return _c.byref(self.xccl)
+
+
+# ---- dispatcher mirror (reference src/utils/mem_component.c) ----------------
+
+def xccl_mem_component_init(path: str = LIB_DIR) -> Status:
+    return _st(dispatch_lib().xccl_mem_component_init(path.encode()))
+
+
+def xccl_mem_component_alloc(nbytes: int, mem_type):
+    p = _vp()
+    st = dispatch_lib().xccl_mem_component_alloc(_c.byref(p), nbytes, int(mem_type))
+    return _st(st), p.value
+
+
+def xccl_mem_component_free(ptr, mem_type) -> Status:
+    return _st(dispatch_lib().xccl_mem_component_free(ptr, int(mem_type)))
+
+
+def xccl_mem_component_type(ptr):
+    mt = _int(-1)
+    st = dispatch_lib().xccl_mem_component_type(ptr, _c.byref(mt))
+    return _st(st), MemType(mt.value)
+
+
+def xccl_mem_component_reduce(sbuf1, sbuf2, target, count, dtype, op, mem_type) -> Status:
+    return _st(dispatch_lib().xccl_mem_component_reduce(sbuf1, sbuf2, target, count, int(dtype), int(op),
+                                                        int(mem_type)))
+
+
+def xccl_mem_component_reduce_multi(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, mem_type) -> Status:
+    return _st(dispatch_lib().xccl_mem_component_reduce_multi(sbuf1, sbuf2, rbuf, count, size, stride, int(dtype),
+                                                              int(op), int(mem_type)))
+
+
+def xccl_mem_component_reduce_nb(sbuf1, sbuf2, target, count, dtype, op, mem_type, stream=None, want_event=True):
+    ev = _vp()
+    st = dispatch_lib().xccl_mem_component_reduce_nb(sbuf1, sbuf2, target, count, int(dtype), int(op), int(mem_type),
+                                                     stream.ref() if stream else None,
+                                                     _c.byref(ev) if want_event else None)
+    return _st(st), ev.value
+
+
+def xccl_mem_component_reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, mem_type, stream=None,
+                                       want_event=True):
+    ev = _vp()
+    st = dispatch_lib().xccl_mem_component_reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, int(dtype),
+                                                           int(op), int(mem_type),
+                                                           stream.ref() if stream else None,
+                                                           _c.byref(ev) if want_event else None)
+    return _st(st), ev.value
+
+
+def xccl_mem_component_memcpy_async(sbuf, dbuf, size, stream: Stream) -> Status:
+    return _st(dispatch_lib().xccl_mem_component_memcpy_async(sbuf, dbuf, size, stream.ref()))
+
+
+def xccl_mem_component_start_acitivity(stream: Stream):
+    req = _vp()
+    st = dispatch_lib().xccl_mem_component_start_acitivity(stream.ref(), _c.byref(req))
+    return _st(st), req.value
+
+
+def xccl_mem_component_finish_acitivity(req) -> Status:
+    return _st(dispatch_lib().xccl_mem_component_finish_acitivity(req))
+
+
+def xccl_mc_event_record(stream: Stream):
+    ev = _vp()
+    st = dispatch_lib().xccl_mc_event_record(stream.ref(), _c.byref(ev))
+    return _st(st), ev.value
+
+
+def xccl_mc_event_query(ev) -> Status:
+    return _st(dispatch_lib().xccl_mc_event_query(ev))
+
+
+def xccl_mc_event_free(ev) -> Status:
+    return _st(dispatch_lib().xccl_mc_event_free(ev))
+
+
+def xccl_mc_event_wait(ev) -> Status:
+    return _st(dispatch_lib().xccl_mc_event_wait(ev))
+
+
+def xccl_mem_component_free_cache():
+    dispatch_lib().xccl_mem_component_free_cache()
+
+
+def xccl_mem_component_finalize():
+    dispatch_lib().xccl_mem_component_finalize()
+
+
+def component_stream():
+    """hipStream_t (int) the component's synchronous entries launch on."""
+    s = _vp()
+    st = component().get_stream(_c.byref(s))
+    if st != 0:
+        raise RuntimeError("get_stream failed: %s" % _st(st))
+    return s.value
+
+
+def datagen_fill(dptr, count, dtype, seed, vec, sparse=False, hip_stream=None) -> Status:
+    return _st(benchkit_lib().xccl_rocm_datagen_fill(dptr, count, int(dtype), seed, vec, int(bool(sparse)),
+                                                    hip_stream))
+
+
+LATENCY_MODES = {"sync": 0, "event": 1, "graph": 2, "stream": 3}
+
+
+def bench_latency(mode: str, sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters: int):
+    """Per-call host-observed durations in ns (numpy uint64) of `iters`
+    back-to-back reduce_multi calls; see csrc/bench_loops.c for the modes."""
+    import numpy as np
+    out = np.zeros(iters, dtype=np.uint64)
+    comp = _c.addressof(component())
+    graph_fn = _c.cast(component_lib().xccl_rocm_reduce_multi_graph, _vp)
+    st = benchkit_lib().xccl_rocm_bench_latency(comp, graph_fn, LATENCY_MODES[mode], sbuf1, sbuf2, rbuf, count, size,
+                                                stride, int(dtype), int(op), iters, out.ctypes.data)
+    return _st(st), out
+
+
+def bench_kernel_times(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters: int):
+    """Device-side duration in ms (numpy float32) of each of `iters` launches,
+    from HIP event pairs recorded on the component stream around each launch."""
+    import numpy as np
+    from . import hip
+    evs = (_vp * (2 * iters))(*[hip.event_create() for _ in range(2 * iters)])
+    out = np.zeros(iters, dtype=np.float32)
+    st = benchkit_lib().xccl_rocm_bench_kernel_times(_c.addressof(component()), sbuf1, sbuf2, rbuf, count, size, stride,
+                                                     int(dtype), int(op), iters, evs, out.ctypes.data)
+    for e in evs:
+        hip.event_destroy(e)
+    return _st(st), out
