@@ -21,9 +21,12 @@
  *     FLOAT16/32/64 (MAX, MIN, SUM, PROD); everything else returns
  *     XCCL_ERR_UNSUPPORTED (the reference kernels' convention).
  *
- * No pointer needs any alignment beyond what the caller already has; rbuf /
- * target may be exactly equal to any one source vector (in-place), and must
- * not overlap a source in any other way.
+ * No pointer needs any alignment beyond what the caller already has.  rbuf /
+ * target may be exactly sbuf1 or exactly sbuf2 (vector 0) -- the two in-place
+ * forms the UCX team library uses (allreduce_knomial.c:118-121,
+ * reduce_linear.c:28-34) -- and must not overlap a source in any other way
+ * (the reference accumulates in rbuf, so with rbuf on a later vector of sbuf2
+ * it reads its own partial result; that artefact is not reproduced).
  */
 #ifndef XCCL_ROCM_KERNELS_H_
 #define XCCL_ROCM_KERNELS_H_
@@ -68,14 +71,16 @@ xccl_status_t xccl_rocm_reduce_multi_graph(void *sbuf1, void *sbuf2, void *rbuf,
 void xccl_rocm_graph_cache_destroy(void);
 
 /*
- * Launch-shape knobs, for measurement.  `blocks_per_cu` caps the persistent
- * grid at blocks_per_cu x (compute units); 0 restores the built-in default.
- * `nontemporal` != 0 selects kernels whose loads/stores carry the
- * non-temporal hint.  Both are process-global and may also be set through
- * the environment (XCCL_MC_ROCM_BLOCKS_PER_CU, XCCL_MC_ROCM_NONTEMPORAL),
- * read once at first launch.
+ * Launch-shape knobs, for measurement.  `blocks_per_cu` caps the grid at
+ * blocks_per_cu x (compute units) workgroups of one wavefront; beyond the cap
+ * workgroups loop over tiles.  0 restores the built-in default (a cap large
+ * enough that every tile gets its own workgroup).  `cache_policy`: 1 =
+ * streaming accesses (non-temporal loads, system-scope stores; the default),
+ * 0 = default-policy loads and stores.  Both are process-global and may also
+ * be set through the environment (XCCL_MC_ROCM_BLOCKS_PER_CU,
+ * XCCL_MC_ROCM_CACHE_POLICY), read once at first launch.
  */
-void xccl_rocm_set_launch_shape(int blocks_per_cu, int nontemporal);
+void xccl_rocm_set_launch_shape(int blocks_per_cu, int cache_policy);
 
 /* What a launch with these arguments would be: grid/block size and the
  * mangled kernel name (truncated into `name`, if not NULL).  Host-only apart

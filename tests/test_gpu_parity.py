@@ -56,13 +56,14 @@ def test_misaligned_pointers_and_odd_strides(rocm, oracle, dt):
                                   (Dt.FLOAT64, Op.PROD), (Dt.UINT16, Op.MIN)], ids=_id)
 def test_in_place(rocm, oracle, pair):
     """rbuf == sbuf1 (allreduce_knomial.c:118-121 after the first round),
-    rbuf == one vector of sbuf2 (reduce_linear.c:28-34: target == sbuf2)."""
+    rbuf == sbuf2{0} (reduce_linear.c:28-34: target == sbuf2).  rbuf equal to
+    a LATER vector of sbuf2 is not a defined use: the reference accumulates in
+    rbuf itself, so that vector is overwritten before it is read."""
     dt, op = pair
     for size in (5, 1024, 10007):
         for n2 in (1, 3, 5, 7):
             run_and_check(rocm, oracle, dt, op, size, n2, alias="s1", seed=5)
             run_and_check(rocm, oracle, dt, op, size, n2, alias=("s2", 0), seed=6)
-            run_and_check(rocm, oracle, dt, op, size, n2, alias=("s2", n2 - 1), seed=7)
 
 
 def test_reference_known_answer_on_device(rocm):
@@ -199,13 +200,13 @@ def test_grid_cap_and_ragged_tiles(rocm, oracle):
     lib = rocm.component_lib()
     try:
         for bpc in (1, 64):
-            lib.xccl_rocm_set_launch_shape(bpc, 0)
+            lib.xccl_rocm_set_launch_shape(bpc, 1)
             for size in (256 * 4 * 2 * 256 + 13, 1 << 20, (1 << 20) + 4 * 255 + 3):
                 run_and_check(rocm, oracle, Dt.FLOAT32, Op.SUM, size, 7, seed=9, check_untouched=False)
                 run_and_check(rocm, oracle, Dt.INT8, Op.SUM, size, 2, seed=9, check_untouched=False)
-        lib.xccl_rocm_set_launch_shape(0, 1)   # kernels with the non-temporal hint
+        lib.xccl_rocm_set_launch_shape(0, 0)   # default-policy loads and stores instead of streaming ones
         for dt, op in ((Dt.FLOAT32, Op.SUM), (Dt.INT16, Op.MAX), (Dt.FLOAT64, Op.MIN)):
             run_and_check(rocm, oracle, dt, op, (1 << 18) + 77, 7, seed=10)
             run_and_check(rocm, oracle, dt, op, 1001, 4, off1=dt_size(dt), seed=10)
     finally:
-        lib.xccl_rocm_set_launch_shape(0, 0)
+        lib.xccl_rocm_set_launch_shape(0, 1)

@@ -14,10 +14,12 @@ namespace xccl_rocm {
 namespace {
 
 constexpr int kMaxDevices       = 64;
-constexpr int kDefaultBlocksPerCu = 8; // 8 x 256 lanes = every wave slot of a CU
+// Grid cap in workgroups per compute unit.  Large on purpose: one tile per
+// workgroup measured fastest, so the cap only bounds the grid of huge calls.
+constexpr int kDefaultBlocksPerCu = 8192;
 
 std::atomic<int> g_blocks_per_cu{-1}; // -1: not read from the environment yet
-std::atomic<int> g_nontemporal{-1};
+std::atomic<int> g_policy{-1};
 std::atomic<int> g_cu_count[kMaxDevices];
 
 void read_env_once()
@@ -25,10 +27,10 @@ void read_env_once()
     if (g_blocks_per_cu.load(std::memory_order_acquire) >= 0) {
         return;
     }
-    const char *nt  = getenv("XCCL_MC_ROCM_NONTEMPORAL");
+    const char *pol = getenv("XCCL_MC_ROCM_CACHE_POLICY");
     const char *bpc = getenv("XCCL_MC_ROCM_BLOCKS_PER_CU");
     int         v   = bpc ? atoi(bpc) : 0;
-    g_nontemporal.store((nt && atoi(nt) != 0) ? 1 : 0, std::memory_order_release);
+    g_policy.store((pol && atoi(pol) == POL_PLAIN) ? POL_PLAIN : POL_STREAM, std::memory_order_release);
     g_blocks_per_cu.store(v > 0 ? v : kDefaultBlocksPerCu, std::memory_order_release);
 }
 
@@ -193,7 +195,7 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
         grid = 1; // head/tail only
     }
     plan->grid = (unsigned)grid;
-    plan->fn   = e->fn[g_nontemporal.load(std::memory_order_relaxed) ? 1 : 0][nv];
+    plan->fn   = e->fn[g_policy.load(std::memory_order_relaxed) == POL_PLAIN ? POL_PLAIN : POL_STREAM][nv];
     return XCCL_OK;
 }
 
@@ -401,11 +403,11 @@ void xccl_rocm_graph_cache_destroy(void)
     }
 }
 
-void xccl_rocm_set_launch_shape(int blocks_per_cu, int nontemporal)
+void xccl_rocm_set_launch_shape(int blocks_per_cu, int cache_policy)
 {
     read_env_once();
     g_blocks_per_cu.store(blocks_per_cu > 0 ? blocks_per_cu : kDefaultBlocksPerCu, std::memory_order_release);
-    g_nontemporal.store(nontemporal ? 1 : 0, std::memory_order_release);
+    g_policy.store(cache_policy == POL_PLAIN ? POL_PLAIN : POL_STREAM, std::memory_order_release);
 }
 
 xccl_status_t xccl_rocm_reduce_multi_plan(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,

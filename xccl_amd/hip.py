@@ -89,7 +89,10 @@ def memcpy_dtod(dst: int, src: int, nbytes: int):
 
 
 def memset(dptr: int, value: int, nbytes: int):
+    """hipMemset + device synchronize: the fill runs on the null stream and is asynchronous to the
+    host, so without the wait it races with work on non-blocking streams."""
     check(lib().hipMemset(ctypes.c_void_p(dptr), ctypes.c_int(value), ctypes.c_size_t(nbytes)), "hipMemset")
+    device_synchronize()
 
 
 def device_synchronize():
