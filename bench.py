@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 N_SRC = 8
 SIZE = 67108864
-TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "reduce_multi_f32_sum_8x256MiB_hbm_traffic.md")
 
 
 def parse():
@@ -44,6 +44,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-latency", action="store_true", help="skip the small-message sweep")
     ap.add_argument("--latency-iters", type=int, default=2000)
+    ap.add_argument("--profile-mode", action="store_true",
+                    help="for rocprofv3: only K headline launches and K launches of a 1 GiB + 1 GiB copy kernel "
+                         "(the known-traffic calibration), nothing else")
     ap.add_argument("--latency-full", action="store_true",
                     help="all 14 sizes x 10,000 iterations; table to gpurun_out/latency.json")
     return ap.parse_args()
@@ -136,6 +139,21 @@ def main():
     hip.device_synchronize()
     stream = mc.component_stream()
 
+    if a.profile_mode:
+        for _ in range(a.warmup + a.steps):
+            st_, _ = mc.xccl_mem_component_reduce_multi_nb(slab, slab + stride, dst, nsrc - 1, size, stride,
+                                                           Dt.FLOAT32, Op.SUM, MemType.ROCM, None, want_event=False)
+            assert st_ == Status.OK
+        hip.stream_synchronize(stream)
+        gib = 1 << 30
+        for _ in range(a.warmup + a.steps):     # sources 0-3 -> sources 4-7: reads 1 GiB, writes 1 GiB
+            assert mc.bench_copy(slab + 4 * stride, slab, gib, stream) == Status.OK
+        hip.stream_synchronize(stream)
+        print(json.dumps({"profile_mode": True, "reduce_launches": a.warmup + a.steps,
+                          "copy_launches": a.warmup + a.steps, "copy_bytes_read": gib, "copy_bytes_written": gib,
+                          "reduce_algorithmic_bytes": nbytes}))
+        return 0
+
     def step():
         st_, _ = mc.xccl_mem_component_reduce_multi_nb(slab, slab + stride, dst, nsrc - 1, size, stride, Dt.FLOAT32,
                                                        Op.SUM, MemType.ROCM, None, want_event=False)
@@ -169,10 +187,10 @@ def main():
     achieved = nbytes / (k_avg * 1e-3) / 1e9
     traffic = None
     if os.path.isfile(TRAFFIC_FILE) and size == SIZE and nsrc == N_SRC:
-        try:
-            traffic = json.load(open(TRAFFIC_FILE)).get("bytes_per_launch")
-        except Exception:
-            traffic = None
+        # measured once with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (the file gives the commands)
+        for line in open(TRAFFIC_FILE):
+            if line.strip().startswith("bytes_per_launch:"):
+                traffic = int(float(line.split(":")[1]))
     # Supplementary: the same call cycling through 4 destination vectors (1 GiB), so that the
     # 256 MiB destination cannot stay resident in the 256 MB Infinity Cache between launches.
     rot = None

@@ -70,7 +70,36 @@ hipError_t fill(void *dst, size_t count, uint64_t base, int sparse, hipStream_t 
     return hipGetLastError();
 }
 
+// A plain 16-byte-per-lane copy: the known-traffic kernel that hardware
+// counter readings are calibrated against (reads n bytes, writes n bytes).
+__global__ void __launch_bounds__(256) copy_kernel(const uint4 *src, uint4 *dst, size_t nvec)
+{
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += step) {
+        dst[i] = src[i];
+    }
+}
+
 } // namespace
+
+// Copies `bytes` (a multiple of 16) from src to dst with copy_kernel on `hip_stream`.
+extern "C" xccl_status_t xccl_rocm_bench_copy(void *dst, const void *src, size_t bytes, void *hip_stream)
+{
+    if (bytes % 16 != 0) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    const size_t nvec   = bytes / 16;
+    size_t       blocks = (nvec + 255) / 256;
+    if (blocks > (1u << 20)) {
+        blocks = 1u << 20;
+    }
+    if (blocks == 0) {
+        return XCCL_OK;
+    }
+    hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)hip_stream, (const uint4 *)src,
+                       (uint4 *)dst, nvec);
+    return hipGetLastError() == hipSuccess ? XCCL_OK : XCCL_ERR_NO_MESSAGE;
+}
 
 // Fills dst[0 .. count) with vector `vec` of the stream identified by `seed`.
 // Enqueues on `hip_stream` (hipStream_t as void*) and returns.

@@ -144,6 +144,7 @@ def benchkit_lib():
         _need_built()
         lib = _c.CDLL(BENCHKIT_SO)
         lib.xccl_rocm_datagen_fill.argtypes = [_vp, _sz, _int, _c.c_uint64, _c.c_uint64, _int, _vp]
+        lib.xccl_rocm_bench_copy.argtypes = [_vp, _vp, _sz, _vp]
         lib.xccl_rocm_bench_latency.argtypes = [_vp, _vp, _int, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
         lib.xccl_rocm_bench_kernel_times.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp]
         _datagen_lib = lib
@@ -274,6 +275,10 @@ def component_stream():
 def datagen_fill(dptr, count, dtype, seed, vec, sparse=False, hip_stream=None) -> Status:
     return _st(benchkit_lib().xccl_rocm_datagen_fill(dptr, count, int(dtype), seed, vec, int(bool(sparse)),
                                                     hip_stream))
+
+
+def bench_copy(dst, src, nbytes, hip_stream=None) -> Status:
+    return _st(benchkit_lib().xccl_rocm_bench_copy(dst, src, nbytes, hip_stream))
 
 
 LATENCY_MODES = {"sync": 0, "event": 1, "graph": 2, "stream": 3}
