@@ -47,6 +47,9 @@ def parse():
     ap.add_argument("--profile-mode", action="store_true",
                     help="for rocprofv3: only K headline launches and K launches of a 1 GiB + 1 GiB copy kernel "
                          "(the known-traffic calibration), nothing else")
+    ap.add_argument("--matrix", action="store_true",
+                    help="kernel GB/s of every BASELINE configuration (all dtype/op pairs of configs 3 and 4 "
+                         "included); table to gpurun_out/matrix.json, nothing else")
     ap.add_argument("--latency-full", action="store_true",
                     help="all 14 sizes x 10,000 iterations; table to gpurun_out/latency.json")
     return ap.parse_args()
@@ -111,6 +114,50 @@ def latency_sweep(mc, hip, iters, full):
     return res
 
 
+def matrix(mc, hip):
+    """Event-timed kernel bandwidth of each BASELINE configuration at its full size."""
+    from xccl_amd.types import Dt, MemType, Op, Status, dt_size, INT_OPS
+    cases = [("config1", Dt.FLOAT32, Op.SUM, 2, 1048576)]
+    cases += [("config2", Dt.FLOAT32, Op.SUM, 8, 67108864)]
+    for dt in (Dt.INT8, Dt.INT16, Dt.INT32, Dt.INT64, Dt.UINT32, Dt.UINT64):
+        cases += [("config3", dt, op, 4, 16777216) for op in INT_OPS]
+    for dt in (Dt.FLOAT16, Dt.FLOAT64):
+        cases += [("config4", dt, op, 16, 33554432) for op in (Op.SUM, Op.MAX, Op.MIN)]
+    cases += [("extra", Dt.FLOAT32, Op.SUM, n, 67108864) for n in (2, 3, 4, 5, 16)]
+    cases += [("extra", Dt.UINT8, op, 4, 67108864) for op in (Op.SUM, Op.MAX)]
+    cases += [("extra", Dt.FLOAT16, Op.PROD, 8, 67108864), ("extra", Dt.FLOAT32, Op.MAX, 8, 67108864)]
+    rows = []
+    cur = None
+    for name, dt, op, nsrc, size in cases:
+        es = dt_size(dt)
+        stride = size * es
+        key = (dt, nsrc, size, op in (Op.LAND, Op.LOR, Op.LXOR))
+        if key != cur:
+            if cur is not None:
+                mc.xccl_mem_component_free(buf, MemType.ROCM)
+            st, buf = mc.xccl_mem_component_alloc((nsrc + 1) * stride, MemType.ROCM)
+            assert st == Status.OK
+            for j in range(nsrc):
+                assert mc.datagen_fill(buf + j * stride, size, dt, 3, j, key[3]) == Status.OK
+            hip.device_synchronize()
+            cur = key
+        st, k = mc.bench_kernel_times(buf, buf + stride, buf + nsrc * stride, nsrc - 1, size, stride, dt, op, 12)
+        assert st == Status.OK
+        ms = float(np.mean(k[2:]))
+        nb = (nsrc + 1) * size * es
+        rows.append({"config": name, "dtype": dt.name, "op": op.name, "nsrc": nsrc, "size": size, "bytes": nb,
+                     "kernel_ms": round(ms, 4), "GBps": round(nb / ms / 1e6, 1),
+                     "frac_of_peak": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 3)})
+        print("%-8s %-8s %-5s N=%-2d size=%-9d %8.4f ms %8.1f GB/s" % (name, dt.name, op.name, nsrc, size, ms,
+                                                                      rows[-1]["GBps"]), file=sys.stderr, flush=True)
+    mc.xccl_mem_component_free(buf, MemType.ROCM)
+    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+    json.dump(rows, open(os.path.join(ROOT, "gpurun_out", "matrix.json"), "w"), indent=1)
+    print(json.dumps({"matrix_rows": len(rows), "min_GBps": min(r["GBps"] for r in rows if r["config"] != "config1"),
+                      "file": "gpurun_out/matrix.json"}))
+    return 0
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -127,6 +174,9 @@ def main():
     hip.set_device(0)
     assert mc.xccl_mem_component_init() == Status.OK
     assert bool(mc.dispatch_lib().xccl_mem_component_get(int(MemType.ROCM))), "ROCm component not loaded"
+
+    if a.matrix:
+        return matrix(mc, hip)
 
     size, nsrc = a.size, a.nsrc
     stride = size * 4

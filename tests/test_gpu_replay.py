@@ -1,0 +1,208 @@
+"""The UCX team library's reduction call sites, replayed over loopback ranks on
+one GPU (libxccl_ucx_replay.so), in the shape of the reference's device tests:
+test/test_mpi_cuda_allreduce.c (INT32 SUM, count 32, rank r contributes
+r + 1 + 12345 + i, compare with the MPI result) and test/test_mpi_cuda_reduce.c
+(the same for every root)."""
+import numpy as np
+import pytest
+
+from gpu_util import NP
+from xccl_amd import hip
+from xccl_amd.types import Dt, Op, Status, dt_size
+
+pytestmark = pytest.mark.gpu
+
+ALLREDUCE = ("allreduce_knomial", "allreduce_sra")
+REDUCE = ("reduce_knomial", "reduce_linear")
+
+
+class Ranks:
+    """P ranks, each with a source and a destination vector in device memory."""
+
+    def __init__(self, host_src: np.ndarray, in_place=False, canary=0xA5):
+        self.P, self.count = host_src.shape
+        self.nbytes = host_src[0].nbytes
+        self.src = [hip.DeviceBuffer(self.nbytes) for _ in range(self.P)]
+        self.dst = self.src if in_place else [hip.DeviceBuffer(self.nbytes) for _ in range(self.P)]
+        for r in range(self.P):
+            self.src[r].upload(host_src[r])
+            if not in_place:
+                hip.memset(self.dst[r].ptr, canary, self.nbytes)
+        self.dtype = host_src.dtype
+
+    def src_ptrs(self):
+        return [b.ptr for b in self.src]
+
+    def dst_ptrs(self):
+        return [b.ptr for b in self.dst]
+
+    def result(self, r):
+        return self.dst[r].download(self.dtype, self.count)
+
+    def source(self, r):
+        return self.src[r].download(self.dtype, self.count)
+
+    def close(self):
+        for b in set(self.src) | set(self.dst):
+            b.close()
+
+
+def _kat(P, count=32):
+    return np.array([[r + 1 + 12345 + i for i in range(count)] for r in range(P)], dtype=np.int32)
+
+
+@pytest.mark.parametrize("alg", ALLREDUCE)
+@pytest.mark.parametrize("stream_ordered", [False, True], ids=["blocking", "stream_ordered"])
+def test_allreduce_known_answer_every_team_size(rocm, alg, stream_ordered):
+    """test_mpi_cuda_allreduce.c:35-76 / test_mt.c:58 for team sizes 2..17 and
+    radices 2..8: every rank must end with P(P+1)/2 + P(i + 12345)."""
+    for P in range(2, 18):
+        expect = [P * (P + 1) // 2 + P * (i + 12345) for i in range(32)]
+        for radix in (2, 3, 4, 5, 8):
+            rk = Ranks(_kat(P))
+            st, stats = rocm.replay_run(alg, rk.src_ptrs(), rk.dst_ptrs(), 32, Dt.INT32, Op.SUM, radix=radix,
+                                        stream_ordered=stream_ordered)
+            assert st == Status.OK, (alg, P, radix, st)
+            for r in range(P):
+                assert rk.result(r).tolist() == expect, (alg, P, radix, r)
+                assert rk.source(r).tolist() == _kat(P)[r].tolist(), "source buffer modified"
+            assert stats["reduce_multi_calls"] > 0 and stats["messages"] > 0
+            rk.close()
+
+
+@pytest.mark.parametrize("alg", REDUCE)
+@pytest.mark.parametrize("stream_ordered", [False, True], ids=["blocking", "stream_ordered"])
+def test_reduce_known_answer_every_root(rocm, alg, stream_ordered):
+    """test_mpi_cuda_reduce.c:47-78: all roots; only the root's destination is
+    written, the others keep their canary."""
+    for P in (2, 3, 4, 5, 7, 8, 9, 16, 17):
+        expect = [P * (P + 1) // 2 + P * (i + 12345) for i in range(32)]
+        for radix in (2, 4, 5):
+            for root in range(P):
+                rk = Ranks(_kat(P))
+                st, stats = rocm.replay_run(alg, rk.src_ptrs(), rk.dst_ptrs(), 32, Dt.INT32, Op.SUM, radix=radix,
+                                            root=root, stream_ordered=stream_ordered)
+                assert st == Status.OK, (alg, P, radix, root, st)
+                assert rk.result(root).tolist() == expect, (alg, P, radix, root)
+                for r in range(P):
+                    if r != root:
+                        assert (rk.result(r).view(np.uint8) == 0xA5).all(), "non-root destination written"
+                if alg == "reduce_linear":
+                    assert stats["reduce_calls"] == P - 1 and stats["inplace_sbuf2"] == P - 1
+                rk.close()
+
+
+def _random_ranks(oracle, P, count, dt, seed):
+    return np.stack([oracle.fill(count, dt, seed, r) for r in range(P)])
+
+
+@pytest.mark.parametrize("alg", ALLREDUCE + REDUCE)
+def test_order_independent_operators_and_ragged_sizes(rocm, oracle, alg):
+    """Integer SUM (wrapping), BXOR, MAX, MIN and LOR give the same bits in any
+    fold order, so numpy's reduction over the rank axis is the expected value
+    whatever tree the algorithm builds.  Counts that do not divide by the radix
+    exercise the uneven scatter-reduce segments."""
+    cases = [(Dt.INT32, Op.SUM, np.add), (Dt.UINT8, Op.BXOR, np.bitwise_xor), (Dt.INT16, Op.MAX, np.maximum),
+             (Dt.UINT64, Op.MIN, np.minimum), (Dt.INT64, Op.SUM, np.add), (Dt.FLOAT64, Op.MAX, np.maximum),
+             (Dt.FLOAT16, Op.MIN, np.minimum)]
+    for P, radix in ((3, 2), (4, 4), (6, 4), (7, 3), (8, 4), (9, 4), (13, 5), (16, 4), (17, 8)):
+        for count in (1, 5, 33, 1000, 4099):
+            dt, op, fn = cases[(P + count) % len(cases)]
+            host = _random_ranks(oracle, P, count, dt, seed=P * 1000 + count)
+            with np.errstate(over="ignore"):
+                want = fn.reduce(host, axis=0, dtype=host.dtype)   # keep the element width: integer SUM wraps
+            rk = Ranks(host)
+            st, stats = rocm.replay_run(alg, rk.src_ptrs(), rk.dst_ptrs(), count, dt, op, radix=radix, root=P // 2)
+            assert st == Status.OK, (alg, P, radix, count, st)
+            who = range(P) if alg in ALLREDUCE else [P // 2]
+            for r in who:
+                assert rk.result(r).tobytes() == want.tobytes(), (alg, P, radix, count, Dt(dt).name, Op(op).name, r)
+            rk.close()
+
+
+@pytest.mark.parametrize("alg", ALLREDUCE)
+def test_in_place_allreduce(rocm, oracle, alg):
+    """src == dst on every rank: the scatter-reduce must move its work space
+    out of dst (allreduce_sra.c:178-186); the k-nomial rounds then alias rbuf
+    with sbuf1 from the first round on."""
+    for P, radix, count in ((4, 4, 1000), (6, 4, 4099), (8, 2, 257), (9, 4, 100000)):
+        host = _random_ranks(oracle, P, count, Dt.INT32, seed=77 + P)
+        want = np.add.reduce(host, axis=0, dtype=host.dtype)
+        rk = Ranks(host, in_place=True)
+        st, stats = rocm.replay_run(alg, rk.src_ptrs(), rk.dst_ptrs(), count, Dt.INT32, Op.SUM, radix=radix)
+        assert st == Status.OK
+        for r in range(P):
+            assert np.array_equal(rk.result(r), want), (alg, P, radix, count, r)
+        assert stats["inplace_sbuf1"] + stats["inplace_sbuf2"] > 0
+        rk.close()
+
+
+@pytest.mark.parametrize("alg", ALLREDUCE + REDUCE)
+def test_float_sum_within_bound_and_exact_on_integers(rocm, oracle, alg):
+    """fp32 SUM: the fold order depends on the algorithm (as it does across
+    ranks in the reference), so random values are checked against a float64
+    sum with |err| <= (P-1) * 2^-24 * sum|x_i|; small integers are exact in
+    every order."""
+    P, radix, count = 8, 4, 50000
+    host = _random_ranks(oracle, P, count, Dt.FLOAT32, seed=5)
+    exact = host.astype(np.float64).sum(axis=0)
+    bound = (P - 1) * 2.0 ** -24 * np.abs(host.astype(np.float64)).sum(axis=0)
+    rk = Ranks(host)
+    st, _ = rocm.replay_run(alg, rk.src_ptrs(), rk.dst_ptrs(), count, Dt.FLOAT32, Op.SUM, radix=radix, root=3)
+    assert st == Status.OK
+    for r in (range(P) if alg in ALLREDUCE else [3]):
+        assert (np.abs(rk.result(r).astype(np.float64) - exact) <= bound).all()
+    rk.close()
+    ints = (_random_ranks(oracle, P, count, Dt.INT8, seed=6).astype(np.float32))
+    rk = Ranks(ints)
+    st, _ = rocm.replay_run(alg, rk.src_ptrs(), rk.dst_ptrs(), count, Dt.FLOAT32, Op.SUM, radix=radix, root=3)
+    assert st == Status.OK
+    for r in (range(P) if alg in ALLREDUCE else [3]):
+        assert np.array_equal(rk.result(r), ints.sum(axis=0, dtype=np.float32))
+    rk.close()
+
+
+def test_call_shapes_of_a_radix4_team_of_8(rocm):
+    """What the state machines ask of the component, counted: 8 ranks, radix 4
+    -> two k-nomial rounds; round one folds 3 received vectors into the own
+    one, round two folds 1 (allreduce_knomial.c:129-135: n = active_reqs/2)."""
+    P, count = 8, 4096
+    rk = Ranks(np.ones((P, count), dtype=np.int32))
+    st, stats = rocm.replay_run("allreduce_knomial", rk.src_ptrs(), rk.dst_ptrs(), count, Dt.INT32, Op.SUM, radix=4)
+    assert st == Status.OK
+    assert stats["reduce_multi_calls"] == 16 and stats["reduce_calls"] == 0 and stats["max_multi_vectors"] == 3
+    assert stats["inplace_sbuf1"] == 8            # second round: rbuf == sbuf1 == dst
+    assert stats["messages"] == 8 * 3 + 8 * 1 and stats["scratch_allocs"] == 8
+    assert (rk.result(5) == P).all()
+    rk.close()
+    # scatter-reduce: round one leaves the result at the start of the work space, which is where the
+    # first arrival sits (rbuf == sbuf2); message bytes shrink by the radix per round
+    rk = Ranks(np.ones((P, count), dtype=np.int32))
+    st, stats = rocm.replay_run("allreduce_sra", rk.src_ptrs(), rk.dst_ptrs(), count, Dt.INT32, Op.SUM, radix=4)
+    assert st == Status.OK and stats["reduce_multi_calls"] == 16 and stats["inplace_sbuf2"] >= 8
+    assert stats["scratch_allocs"] == 0           # dst doubles as work space when src != dst
+    assert (rk.result(2) == P).all()
+    rk.close()
+    # 6 ranks: 2 extras hand their vectors to proxies, who fold them in with a 2-source reduce first
+    rk = Ranks(np.ones((6, count), dtype=np.int32))
+    st, stats = rocm.replay_run("allreduce_knomial", rk.src_ptrs(), rk.dst_ptrs(), count, Dt.INT32, Op.SUM, radix=4)
+    assert st == Status.OK and stats["reduce_calls"] == 2 and stats["reduce_multi_calls"] == 4
+    assert all((rk.result(r) == 6).all() for r in range(6))
+    rk.close()
+
+
+def test_large_vectors_stream_ordered_overlap(rocm, oracle):
+    """64 MiB per rank, 4 ranks: the reductions take long enough that ranks
+    return with theirs still in flight, and other ranks' progress functions
+    run meanwhile -- the point of the stream-ordered call sites."""
+    P, count = 4, 16 * 1024 * 1024
+    host = _random_ranks(oracle, P, count, Dt.INT32, seed=9)
+    want = np.add.reduce(host, axis=0, dtype=host.dtype)
+    for alg in ALLREDUCE:
+        rk = Ranks(host)
+        st, stats = rocm.replay_run(alg, rk.src_ptrs(), rk.dst_ptrs(), count, Dt.INT32, Op.SUM, radix=4)
+        assert st == Status.OK
+        for r in range(P):
+            assert np.array_equal(rk.result(r), want)
+        assert stats["reduce_inflight_returns"] > 0
+        rk.close()

@@ -6,7 +6,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 
-LIBS = ("xccl_rocm_mem_component.so", "libxccl_mc.so", "libxccl_rocm_benchkit.so")
+LIBS = ("xccl_rocm_mem_component.so", "libxccl_mc.so", "libxccl_rocm_benchkit.so", "libxccl_ucx_replay.so")
 
 
 def built() -> bool:

@@ -66,6 +66,7 @@ class RocmMemComponent(_c.Structure):
 
 COMPONENT_SO = os.path.join(LIB_DIR, "xccl_rocm_mem_component.so")
 DISPATCH_SO = os.path.join(LIB_DIR, "libxccl_mc.so")
+REPLAY_SO = os.path.join(LIB_DIR, "libxccl_ucx_replay.so")
 BENCHKIT_SO = os.path.join(LIB_DIR, "libxccl_rocm_benchkit.so")
 
 _component_lib = None
@@ -308,3 +309,65 @@ def bench_kernel_times(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters
     for e in evs:
         hip.event_destroy(e)
     return _st(st), out
+
+
+# ---- UCX team-library call sites over a loopback transport (include/xccl_rocm_ucx_replay.h) ----
+
+class ReplayParams(_c.Structure):
+    _fields_ = [("alg", _int), ("reduce_mode", _int), ("team_size", _int), ("radix", _int), ("root", _int),
+                ("count", _sz), ("dtype", _int), ("op", _int), ("src", _c.POINTER(_vp)), ("dst", _c.POINTER(_vp))]
+
+
+class ReplayStats(_c.Structure):
+    _fields_ = [(n, _c.c_uint64) for n in (
+        "reduce_calls", "reduce_multi_calls", "max_multi_vectors", "inplace_sbuf1", "inplace_sbuf2", "messages",
+        "bytes_moved", "progress_calls", "reduce_inflight_returns", "scratch_allocs")]
+
+    def as_dict(self):
+        return {n: int(getattr(self, n)) for n, _ in self._fields_}
+
+
+REPLAY_ALGS = {"allreduce_knomial": 0, "allreduce_sra": 1, "reduce_knomial": 2, "reduce_linear": 3}
+_replay_lib = None
+
+
+def replay_lib():
+    global _replay_lib
+    if _replay_lib is None:
+        _need_built()
+        dispatch_lib()
+        lib = _c.CDLL(REPLAY_SO)
+        lib.xccl_replay_run.argtypes = [_c.POINTER(ReplayParams), _c.POINTER(ReplayStats), _c.c_uint64]
+        lib.xccl_replay_knomial_geometry.argtypes = [_int, _int, _int, _c.POINTER(_int), _c.POINTER(_int),
+                                                     _c.POINTER(_int)]
+        lib.xccl_replay_knomial_geometry.restype = None
+        lib.xccl_replay_sra_segment.argtypes = [_sz, _int, _int, _int, _c.POINTER(_sz), _c.POINTER(_sz)]
+        lib.xccl_replay_sra_segment.restype = None
+        _replay_lib = lib
+    return _replay_lib
+
+
+def replay_run(alg: str, src_ptrs, dst_ptrs, count, dtype, op, radix=4, root=0, stream_ordered=True, max_sweeps=0):
+    """One collective over len(src_ptrs) loopback ranks; returns (Status, stats dict)."""
+    n = len(src_ptrs)
+    src = (_vp * n)(*src_ptrs)
+    dst = (_vp * n)(*dst_ptrs)
+    prm = ReplayParams(REPLAY_ALGS[alg], 1 if stream_ordered else 0, n, radix, root, count, int(dtype), int(op),
+                       _c.cast(src, _c.POINTER(_vp)), _c.cast(dst, _c.POINTER(_vp)))
+    stats = ReplayStats()
+    st = replay_lib().xccl_replay_run(_c.byref(prm), _c.byref(stats), max_sweeps)
+    return _st(st), stats.as_dict()
+
+
+def knomial_geometry(radix, rank, team_size):
+    """(rounds, full_size, role) with role 0 = base, 1 = proxy, 2 = extra."""
+    a, b, r = _int(0), _int(0), _int(0)
+    replay_lib().xccl_replay_knomial_geometry(radix, rank, team_size, _c.byref(a), _c.byref(b), _c.byref(r))
+    return a.value, b.value, r.value
+
+
+def sra_segment(count, rank, radix, team_size):
+    """(element offset, length) of the segment `rank` owns after the scatter-reduce."""
+    o, n = _sz(0), _sz(0)
+    replay_lib().xccl_replay_sra_segment(count, rank, radix, team_size, _c.byref(o), _c.byref(n))
+    return o.value, n.value
