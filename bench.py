@@ -15,7 +15,10 @@ before the timed region.  Prints ONE JSON line.
                    launch, against 8 TB/s HBM3E
   cpu_baseline     the CPU oracle (port of the reference's host fold, one
                    thread) timed on this box on the same workload
-  latency_us       small-message p50 per call, FLOAT32 SUM, 2/4/8 sources
+  latency_us       small-message p50/p99 per call in us, FLOAT32 SUM, 2/4/8 sources: "sync" = the blocking
+                   vtable entry, "event" = reduce_multi_nb + event_query polling (both complete through the
+                   kernel's own completion word), "stream" = reduce_multi_nb + hipStreamSynchronize,
+                   "graph" = single-node hipGraph launch + hipStreamSynchronize
 """
 import argparse
 import json
@@ -102,7 +105,7 @@ def latency_sweep(mc, hip, iters, full):
         for b in sizes_b:
             cnt = b // 4
             row = {}
-            for mode in ("sync", "event", "graph"):
+            for mode in ("sync", "event", "stream", "graph"):
                 st, ns = mc.bench_latency(mode, buf.ptr, buf.ptr + maxb, buf.ptr + 9 * maxb, nsrc - 1, cnt, maxb,
                                           Dt.FLOAT32, Op.SUM, iters)
                 assert st == Status.OK, (mode, st)

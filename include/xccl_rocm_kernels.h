@@ -56,6 +56,25 @@ xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf,
                                           size_t stride, xccl_dt_t dtype,
                                           xccl_op_t op, void *hip_stream);
 
+/*
+ * xccl_rocm_reduce_multi_impl with a completion word: when the launch is small
+ * (a few hundred workgroups at most) the kernel itself stores `seq` to
+ * `*dev_flag` -- the device view of a host-mapped 32-bit word -- after its
+ * last result store is visible system-wide, and `*flagged` is set to 1; the
+ * caller may then poll the host view of the word instead of the stream.
+ * `dev_count` is a zeroed 32-bit device word the workgroups count arrivals in;
+ * the kernel leaves it zero again.  One launch at a time per (count, flag)
+ * pair.  For larger launches nothing is attached, `*flagged` is 0 and the
+ * caller waits for the stream as usual.  No counterpart in the reference.
+ */
+xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbuf,
+                                             size_t count, size_t size,
+                                             size_t stride, xccl_dt_t dtype,
+                                             xccl_op_t op, void *hip_stream,
+                                             uint32_t *dev_count,
+                                             uint32_t *dev_flag, uint32_t seq,
+                                             int *flagged);
+
 /* Same contract and same kernel as xccl_rocm_reduce_multi_impl, but enqueued
  * as one launch of a pre-instantiated single-kernel-node hipGraph whose node
  * parameters are patched per call (a small per-device cache keeps the most

@@ -245,3 +245,117 @@ def test_datagen_matches_oracle_generator(rocm, oracle, dt):
         else:
             assert got.tobytes() == want.tobytes()
     d.close()
+
+
+def test_completion_word_threshold_and_sequences(rocm, oracle):
+    """Small launches complete through a host-mapped word the kernel writes,
+    large ones through the stream.  Sizes on both sides of the switch (512
+    workgroups), many back-to-back blocking calls (sequence numbers advance
+    per pooled event), results checked every time."""
+    dt, op = Dt.FLOAT32, Op.SUM
+    for size in (1, 63, 262144 - 1, 262144, 262144 + 1, 262144 + 513, 1 << 20):
+        c = Case(dt, size, 1)
+        try:
+            c.fill_random(oracle, 21)
+            c.upload()
+            p1, p2, pr = c.ptrs()
+            want, _ = c.expect(oracle, op)
+            for rep in range(5):
+                hip.memset(pr, 0x11 * (rep + 1), c.vbytes)
+                assert rocm.xccl_mem_component_reduce_multi(p1, p2, pr, 1, size, c.stride, dt, op,
+                                                            MemType.ROCM) == Status.OK
+                assert_same(c.result(), want, dt, op, "size %d rep %d" % (size, rep))
+        finally:
+            c.close()
+    # 300 blocking calls in a row on a tiny message: every one must be complete on return
+    c = Case(Dt.INT32, 64, 3)
+    try:
+        c.fill_random(oracle, 22)
+        c.upload()
+        p1, p2, pr = c.ptrs()
+        want, _ = c.expect(oracle, Op.SUM)
+        for rep in range(300):
+            assert rocm.xccl_mem_component_reduce_multi(p1, p2, pr, 3, 64, c.stride, Dt.INT32, Op.SUM,
+                                                        MemType.ROCM) == Status.OK
+            if rep % 50 == 0:
+                assert_same(c.result(), want, Dt.INT32, Op.SUM, "rep %d" % rep)
+    finally:
+        c.close()
+
+
+def test_many_events_in_flight_any_wait_order(rocm, oracle):
+    """One pooled event per launch, 48 launches enqueued before the first wait,
+    waited for in reverse order, mixed small (completion word) and large
+    (HIP event) launches; then the pool is whole again."""
+    dt, op = Dt.INT32, Op.BXOR
+    cases, evs = [], []
+    try:
+        for k in range(48):
+            size = (1 << 19) + 5 if k % 6 == 5 else 100 + 17 * k
+            c = Case(dt, size, 1 + k % 3)
+            c.fill_random(oracle, 50 + k)
+            c.upload()
+            cases.append(c)
+        for c in cases:
+            p1, p2, pr = c.ptrs()
+            st, ev = rocm.xccl_mem_component_reduce_multi_nb(p1, p2, pr, c.n2, c.size, c.stride, dt, op, MemType.ROCM)
+            assert st == Status.OK and ev
+            evs.append(ev)
+        for c, ev in reversed(list(zip(cases, evs))):
+            assert rocm.xccl_mc_event_wait(ev) == Status.OK
+            assert rocm.xccl_mc_event_query(ev) == Status.OK
+            want, _ = c.expect(oracle, op)
+            assert_same(c.result(), want, dt, op, "size %d" % c.size)
+            assert rocm.xccl_mc_event_free(ev) == Status.OK
+        s = rocm.Stream(hip.stream_create())
+        got = []
+        while True:
+            st, ev = rocm.xccl_mc_event_record(s)
+            if st != Status.OK:
+                break
+            got.append(ev)
+        assert len(got) == 64
+        for ev in got:
+            rocm.xccl_mc_event_free(ev)
+        hip.stream_destroy(s.hip_stream)
+    finally:
+        for c in cases:
+            c.close()
+
+
+def test_blocking_calls_from_several_threads(rocm, oracle):
+    """test/test_mt.c runs 4 threads of collectives; the component's pools and
+    lazy initialisation must hold up: 4 threads x 200 blocking reductions on
+    private buffers, every result checked."""
+    import threading
+    dt, op, size = Dt.INT32, Op.SUM, 4096
+    cases = []
+    for t in range(4):
+        c = Case(dt, size + t, 3)
+        c.fill_random(oracle, 70 + t)
+        c.upload()
+        cases.append(c)
+    errors = []
+
+    def worker(c):
+        try:
+            p1, p2, pr = c.ptrs()
+            want, _ = c.expect(oracle, op)
+            for rep in range(200):
+                st = rocm.xccl_mem_component_reduce_multi(p1, p2, pr, 3, c.size, c.stride, dt, op, MemType.ROCM)
+                if st != Status.OK:
+                    errors.append(st)
+                    return
+                if rep % 40 == 0:
+                    assert_same(c.result(), want, dt, op, "thread size %d rep %d" % (c.size, rep))
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(c,)) for c in cases]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for c in cases:
+        c.close()
+    assert not errors, errors

@@ -47,11 +47,24 @@
 /* pool slot states (`is_free` keeps the reference's member name) */
 enum { MC_SLOT_BUSY = 0, MC_SLOT_FREE = 1, MC_SLOT_DRAINING = 2 };
 
+/* An event completes either through its HIP event, or -- when it stands for a
+ * small reduction launch -- through a host-mapped word the kernel itself
+ * stores a sequence number to (cheaper to observe than the queue's completion
+ * signal by ~4 us on this part). */
 typedef struct mc_rocm_event {
-    xccl_mc_event_t super;
-    atomic_int      is_free;
-    hipEvent_t      hip_event;
+    xccl_mc_event_t    super;
+    atomic_int         is_free;
+    hipEvent_t         hip_event;
+    int                flagged;   /* 1: done when *flag == expect */
+    uint32_t           expect;    /* last sequence number handed to a kernel */
+    volatile uint32_t *flag;      /* host view of the completion word */
+    uint32_t          *dev_flag;  /* device view of the same word */
+    uint32_t          *dev_count; /* arrival counter of the launch's workgroups */
+    hipStream_t        stream;    /* where the work was enqueued */
+    unsigned           polls;
 } mc_rocm_event_t;
+
+#define MC_FLAG_STRIDE 16 /* uint32 words between completion words: one per 64-byte line */
 
 typedef struct mc_rocm_stream_request {
     xccl_mem_component_stream_request_t super;
@@ -65,6 +78,8 @@ typedef struct mc_rocm_device {
     atomic_int               ready; /* 0 = untouched, 1 = usable */
     hipStream_t              stream;
     int                     *gate_words; /* pinned, mapped */
+    uint32_t                *flag_words; /* pinned, mapped: completion words of the events */
+    uint32_t                *arrival_counts; /* device */
     mc_rocm_event_t          events[XCCL_ROCM_MC_NUM_EVENTS];
     mc_rocm_stream_request_t requests[XCCL_ROCM_MC_NUM_STREAM_REQUESTS];
 } mc_rocm_device_t;
@@ -118,10 +133,24 @@ static xccl_status_t mc_rocm_device_create(mc_rocm_device_t *d)
         MC_HIP(hipEventCreateWithFlags(&r->hip_event, hipEventDisableTiming));
         atomic_store(&r->is_free, 1);
     }
+    MC_HIP(hipHostMalloc((void **)&d->flag_words,
+                         XCCL_ROCM_MC_NUM_EVENTS * MC_FLAG_STRIDE * sizeof(uint32_t),
+                         hipHostMallocMapped));
+    memset(d->flag_words, 0, XCCL_ROCM_MC_NUM_EVENTS * MC_FLAG_STRIDE * sizeof(uint32_t));
+    MC_HIP(hipMalloc((void **)&d->arrival_counts,
+                     XCCL_ROCM_MC_NUM_EVENTS * sizeof(uint32_t)));
+    MC_HIP(hipMemsetAsync(d->arrival_counts, 0,
+                          XCCL_ROCM_MC_NUM_EVENTS * sizeof(uint32_t), d->stream));
+    MC_HIP(hipStreamSynchronize(d->stream));
     for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
-        MC_HIP(hipEventCreateWithFlags(&d->events[i].hip_event,
-                                       hipEventDisableTiming));
-        atomic_store(&d->events[i].is_free, 1);
+        mc_rocm_event_t *ev = &d->events[i];
+        MC_HIP(hipEventCreateWithFlags(&ev->hip_event, hipEventDisableTiming));
+        ev->flag = &d->flag_words[i * MC_FLAG_STRIDE];
+        MC_HIP(hipHostGetDevicePointer((void **)&ev->dev_flag, (void *)ev->flag, 0));
+        ev->dev_count = &d->arrival_counts[i];
+        ev->expect    = 0;
+        ev->flagged   = 0;
+        atomic_store(&ev->is_free, 1);
     }
     return XCCL_OK;
 }
@@ -208,6 +237,33 @@ static xccl_status_t mc_rocm_user_stream(xccl_stream_t *stream, hipStream_t *out
     return XCCL_OK;
 }
 
+/* Completion of a flagged launch, observed from the host.  `block`: spin until
+ * done.  Every 64 Ki polls the stream is asked whether it failed or drained
+ * without the word being written, so a broken launch cannot spin forever. */
+static xccl_status_t mc_rocm_flag_poll(mc_rocm_event_t *ev, int block)
+{
+    hipError_t e;
+
+    for (;;) {
+        if (__atomic_load_n(ev->flag, __ATOMIC_ACQUIRE) == ev->expect) {
+            return XCCL_OK;
+        }
+        if ((++ev->polls & 0xffffu) == 0) {
+            e = hipStreamQuery(ev->stream);
+            if (e == hipSuccess) {
+                return __atomic_load_n(ev->flag, __ATOMIC_ACQUIRE) == ev->expect
+                           ? XCCL_OK : XCCL_ERR_NO_MESSAGE;
+            }
+            if (e != hipErrorNotReady) {
+                return XCCL_ERR_NO_MESSAGE;
+            }
+        }
+        if (!block) {
+            return XCCL_INPROGRESS;
+        }
+    }
+}
+
 /* Shared tail of the four reduction entries.  `want_sync`: block until the
  * result is visible (the vtable's reduce / reduce_multi contract, reference
  * xccl_cuda_reduce_multi.cu:140). */
@@ -223,6 +279,7 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
     mc_rocm_event_t  *ev = NULL;
     hipStream_t       hs;
     xccl_status_t     st;
+    int               flagged = 0;
 
     st = xccl_rocm_reduce_supported(dtype, op);
     if (st != XCCL_OK) {
@@ -239,9 +296,11 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
             return st;
         }
     }
-    if (event != NULL) {
+    if (event != NULL || want_sync) {
+        /* a pooled event brings the completion word; a blocking call can do
+         * without one (then it waits for the stream) */
         ev = mc_rocm_claim_event(d);
-        if (ev == NULL) {
+        if (ev == NULL && event != NULL) {
             return XCCL_ERR_NO_RESOURCE;
         }
     }
@@ -249,29 +308,48 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
     if (want_sync && size * xccl_dt_size(dtype) <= mc_graph_max_bytes) {
         st = xccl_rocm_reduce_multi_graph(sbuf1, sbuf2, rbuf, count, size,
                                           stride, dtype, op, hs);
+    } else if (ev != NULL) {
+        st = xccl_rocm_reduce_multi_flagged(sbuf1, sbuf2, rbuf, count, size,
+                                            stride, dtype, op, hs,
+                                            ev->dev_count, ev->dev_flag,
+                                            ev->expect + 1, &flagged);
     } else {
         st = xccl_rocm_reduce_multi_impl(sbuf1, sbuf2, rbuf, count, size,
                                          stride, dtype, op, hs);
     }
     if (st != XCCL_OK) {
         if (ev != NULL) {
-            atomic_store(&ev->is_free, 1);
+            atomic_store(&ev->is_free, MC_SLOT_FREE);
         }
         return st;
     }
     if (ev != NULL) {
-        hipError_t e = hipEventRecord(ev->hip_event, hs);
-        if (e != hipSuccess) {
-            atomic_store(&ev->is_free, 1);
+        ev->stream  = hs;
+        ev->flagged = flagged;
+        ev->polls   = 0;
+        if (flagged) {
+            ev->expect++;
+        } else if (event != NULL && hipEventRecord(ev->hip_event, hs) != hipSuccess) {
+            atomic_store(&ev->is_free, MC_SLOT_FREE);
             return XCCL_ERR_NO_MESSAGE;
         }
-        ev->super.mem_type = UCS_MEMORY_TYPE_ROCM;
-        *event             = &ev->super;
     }
     if (want_sync) {
-        MC_HIP(hipStreamSynchronize(hs));
+        if (flagged) {
+            st = mc_rocm_flag_poll(ev, 1);
+        } else if (hipStreamSynchronize(hs) != hipSuccess) {
+            st = XCCL_ERR_NO_MESSAGE;
+        }
     }
-    return XCCL_OK;
+    if (ev != NULL) {
+        if (event != NULL && st == XCCL_OK) {
+            ev->super.mem_type = UCS_MEMORY_TYPE_ROCM;
+            *event             = &ev->super;
+        } else {
+            atomic_store(&ev->is_free, MC_SLOT_FREE);
+        }
+    }
+    return st;
 }
 
 static xccl_status_t mc_rocm_reduce(void *sbuf1, void *sbuf2, void *target,
@@ -345,6 +423,8 @@ static xccl_status_t mc_rocm_event_record(xccl_stream_t *stream,
     if (ev == NULL) {
         return XCCL_ERR_NO_RESOURCE;
     }
+    ev->flagged = 0;
+    ev->stream  = hs;
     e = hipEventRecord(ev->hip_event, hs);
     if (e != hipSuccess) {
         atomic_store(&ev->is_free, 1);
@@ -367,6 +447,9 @@ static xccl_status_t mc_rocm_event_query(xccl_mc_event_t *event)
     if (event == NULL) {
         return XCCL_ERR_INVALID_PARAM;
     }
+    if (mc_rocm_event_of(event)->flagged) {
+        return mc_rocm_flag_poll(mc_rocm_event_of(event), 0);
+    }
     e = hipEventQuery(mc_rocm_event_of(event)->hip_event);
     if (e == hipSuccess) {
         return XCCL_OK;
@@ -381,6 +464,9 @@ static xccl_status_t mc_rocm_event_wait(xccl_mc_event_t *event)
 {
     if (event == NULL) {
         return XCCL_ERR_INVALID_PARAM;
+    }
+    if (mc_rocm_event_of(event)->flagged) {
+        return mc_rocm_flag_poll(mc_rocm_event_of(event), 1);
     }
     MC_HIP(hipEventSynchronize(mc_rocm_event_of(event)->hip_event));
     return XCCL_OK;
@@ -501,6 +587,8 @@ static void mc_rocm_close(void)
             (void)hipEventDestroy(d->requests[i].hip_event);
         }
         (void)hipHostFree(d->gate_words);
+        (void)hipHostFree(d->flag_words);
+        (void)hipFree(d->arrival_counts);
         (void)hipStreamDestroy(d->stream);
         memset(d, 0, sizeof(*d));
     }

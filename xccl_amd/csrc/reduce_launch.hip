@@ -118,7 +118,8 @@ bool same_plan(const Plan &a, const Plan &b)
 {
     return a.fn == b.fn && a.grid == b.grid && a.args.s1 == b.args.s1 && a.args.s2 == b.args.s2 &&
            a.args.dst == b.args.dst && a.args.stride == b.args.stride && a.args.head == b.args.head &&
-           a.args.nvec == b.args.nvec && a.args.tail == b.args.tail && a.args.n2 == b.args.n2;
+           a.args.nvec == b.args.nvec && a.args.tail == b.args.tail && a.args.n2 == b.args.n2 &&
+           a.args.done_flag == b.args.done_flag && a.args.done_seq == b.args.done_seq;
 }
 
 // Bytes to peel so that as many of the buffers as possible start their
@@ -186,6 +187,9 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     a.nvec   = (elems - head) / ve;
     a.tail   = (elems - head) % ve;
     a.n2     = n2;
+    a.done_seq   = 0;
+    a.done_count = nullptr;
+    a.done_flag  = nullptr;
 
     const size_t tile  = (size_t)kBlock * unroll_of(nv);
     const size_t tiles = (a.nvec + tile - 1) / tile;
@@ -198,6 +202,11 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     plan->fn   = e->fn[g_policy.load(std::memory_order_relaxed) == POL_PLAIN ? POL_PLAIN : POL_STREAM][nv];
     return XCCL_OK;
 }
+
+// Launches of at most this many workgroups may carry a completion word: each
+// workgroup pays one atomic on a shared counter, which is nothing for a few
+// hundred and would serialise a grid of hundreds of thousands.
+constexpr unsigned kMaxFlaggedGrid = 512;
 
 // ---- single-kernel-node graph cache ---------------------------------------
 constexpr int kGraphSlots = 8;
@@ -357,6 +366,35 @@ xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf, 
     xccl_status_t st = make_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan);
     if (st != XCCL_OK) {
         return st;
+    }
+    void *argv[1] = {&plan.args};
+    HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, 0, (hipStream_t)hip_stream));
+    return XCCL_OK;
+}
+
+xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
+                                             size_t stride, xccl_dt_t dtype, xccl_op_t op, void *hip_stream,
+                                             uint32_t *dev_count, uint32_t *dev_flag, uint32_t seq, int *flagged)
+{
+    if (flagged) {
+        *flagged = 0;
+    }
+    if (lookup(dtype, op) == nullptr) {
+        return XCCL_ERR_UNSUPPORTED;
+    }
+    if (size == 0) {
+        return XCCL_OK;
+    }
+    Plan          plan;
+    xccl_status_t st = make_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    if (dev_count != nullptr && dev_flag != nullptr && flagged != nullptr && plan.grid <= kMaxFlaggedGrid) {
+        plan.args.done_seq   = seq;
+        plan.args.done_count = dev_count;
+        plan.args.done_flag  = dev_flag;
+        *flagged             = 1;
     }
     void *argv[1] = {&plan.args};
     HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, 0, (hipStream_t)hip_stream));
