@@ -51,10 +51,11 @@ def parse():
                     help="for rocprofv3: only K headline launches and K launches of a 1 GiB + 1 GiB copy kernel "
                          "(the known-traffic calibration), nothing else")
     ap.add_argument("--matrix", action="store_true",
-                    help="kernel GB/s of every BASELINE configuration (all dtype/op pairs of configs 3 and 4 "
-                         "included); table to gpurun_out/matrix.json, nothing else")
+                    help="kernel GB/s of every benchmark configuration (all dtype/op pairs of the integer sweep "
+                         "and the 16-source cases included); table to <out-dir>/matrix.json, nothing else")
     ap.add_argument("--latency-full", action="store_true",
-                    help="all 14 sizes x 10,000 iterations; table to gpurun_out/latency.json")
+                    help="all 14 sizes x 10,000 iterations; table to <out-dir>/latency.json")
+    ap.add_argument("--out-dir", default=os.path.join(ROOT, "bench_out"), help="where --matrix / --latency-full write")
     return ap.parse_args()
 
 
@@ -117,8 +118,8 @@ def latency_sweep(mc, hip, iters, full):
     return res
 
 
-def matrix(mc, hip):
-    """Event-timed kernel bandwidth of each BASELINE configuration at its full size."""
+def matrix(mc, hip, out_dir):
+    """Event-timed kernel bandwidth of each benchmark configuration at its full size."""
     from xccl_amd.types import Dt, MemType, Op, Status, dt_size, INT_OPS
     cases = [("config1", Dt.FLOAT32, Op.SUM, 2, 1048576)]
     cases += [("config2", Dt.FLOAT32, Op.SUM, 8, 67108864)]
@@ -154,10 +155,10 @@ def matrix(mc, hip):
         print("%-8s %-8s %-5s N=%-2d size=%-9d %8.4f ms %8.1f GB/s" % (name, dt.name, op.name, nsrc, size, ms,
                                                                       rows[-1]["GBps"]), file=sys.stderr, flush=True)
     mc.xccl_mem_component_free(buf, MemType.ROCM)
-    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-    json.dump(rows, open(os.path.join(ROOT, "gpurun_out", "matrix.json"), "w"), indent=1)
+    os.makedirs(out_dir, exist_ok=True)
+    json.dump(rows, open(os.path.join(out_dir, "matrix.json"), "w"), indent=1)
     print(json.dumps({"matrix_rows": len(rows), "min_GBps": min(r["GBps"] for r in rows if r["config"] != "config1"),
-                      "file": "gpurun_out/matrix.json"}))
+                      "file": os.path.join(out_dir, "matrix.json")}))
     return 0
 
 
@@ -179,7 +180,7 @@ def main():
     assert bool(mc.dispatch_lib().xccl_mem_component_get(int(MemType.ROCM))), "ROCm component not loaded"
 
     if a.matrix:
-        return matrix(mc, hip)
+        return matrix(mc, hip, a.out_dir)
 
     size, nsrc = a.size, a.nsrc
     stride = size * 4
@@ -270,7 +271,7 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "reduce_multi FLOAT32 SUM, %d source vectors x %d elements at stride %d B in one slab "
-                               "(BASELINE configs[1]); stream-ordered launches" % (nsrc, size, stride),
+                               "(radix-8 k-nomial step); stream-ordered launches" % (nsrc, size, stride),
                    "bytes_per_step": nbytes, "device": hip.device_name(0) or "gfx950",
                    "kernel": name.value.decode(), "grid": grid.value, "block": block.value},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
@@ -295,8 +296,8 @@ def main():
     if not a.no_latency:
         lat = latency_sweep(mc, hip, a.latency_iters, a.latency_full)
         if a.latency_full:
-            os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-            json.dump(lat, open(os.path.join(ROOT, "gpurun_out", "latency.json"), "w"), indent=1)
+            os.makedirs(a.out_dir, exist_ok=True)
+            json.dump(lat, open(os.path.join(a.out_dir, "latency.json"), "w"), indent=1)
             out["latency_us"] = {k: v for k, v in lat.items() if k.endswith(("_4B", "_1024B", "_32768B"))}
         else:
             out["latency_us"] = lat

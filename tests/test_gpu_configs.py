@@ -119,3 +119,40 @@ def test_properties_at_full_size(rocm, oracle):
     ok = ~np.isnan(f) & (v != 0x80000000)
     assert np.array_equal(g.view(np.uint32)[ok], v[ok])
     dev.close()
+
+
+def test_vectors_beyond_4GiB(rocm, oracle):
+    """Vectors larger than 2^32 bytes (the device has 288 GB; the scatter-reduce
+    path hands over whatever the user's buffer is): 64-bit indexing end to end.
+    Three 5 GiB float vectors; windows at the start, across the 4 GiB line, and
+    at the ragged end are compared with the oracle run on the same bytes."""
+    size = 5 * (1 << 28) + 3                      # 1,342,177,283 floats = 5 GiB + 12 B
+    stride = (size * 4 + 255) // 256 * 256
+    free_b, _ = hip.mem_get_info()
+    if free_b < 3 * stride + (1 << 30):
+        pytest.skip("not enough free device memory")
+    dev = hip.DeviceBuffer(3 * stride)
+    try:
+        for j in range(2):
+            assert rocm.datagen_fill(dev.ptr + j * stride, size, Dt.FLOAT32, 9, j) == Status.OK
+        hip.device_synchronize()
+        assert rocm.xccl_mem_component_reduce_multi(dev.ptr, dev.ptr + stride, dev.ptr + 2 * stride, 1, size, stride,
+                                                    Dt.FLOAT32, Op.SUM, MemType.ROCM) == Status.OK
+        win = 1 << 18
+        for lo in (0, (1 << 30) - win // 2, size - win):      # element 2^30 sits at byte 2^32
+            a = dev.download(np.float32, win, lo * 4)
+            b = dev.download(np.float32, win, stride + lo * 4)
+            got = dev.download(np.float32, win, 2 * stride + lo * 4)
+            want = np.empty(win, dtype=np.float32)
+            assert oracle.dt_reduce(a, b, want, win, Dt.FLOAT32, Op.SUM) == 0
+            assert got.tobytes() == want.tobytes(), "window at element %d" % lo
+            assert np.count_nonzero(a) > win // 2 and np.count_nonzero(b) > win // 2
+        # byte kernel with three sources, same footprint
+        assert rocm.xccl_mem_component_reduce_multi(dev.ptr, dev.ptr + stride, dev.ptr + 2 * stride, 1, size * 4, stride,
+                                                    Dt.UINT8, Op.BXOR, MemType.ROCM) == Status.OK
+        for lo in ((1 << 32) - 4096, size * 4 - 8192):
+            a = dev.download(np.uint8, 8192, lo)
+            b = dev.download(np.uint8, 8192, stride + lo)
+            assert np.array_equal(dev.download(np.uint8, 8192, 2 * stride + lo), a ^ b)
+    finally:
+        dev.close()

@@ -70,18 +70,20 @@ def test_reference_known_answer_on_device(rocm):
     """test/test_mpi_cuda_allreduce.c:35-39 + test/test_mt.c:58: INT32 SUM,
     count 32, rank r contributes r + 1 + 12345 + i; expect P(P+1)/2 + P(i+12345).
     Rank 0's vector is sbuf1, the others arrive in scratch = sbuf2."""
+    import json
+    import os
     from xccl_amd import hip
-    count = 32
-    for nranks in (2, 3, 4, 5, 8, 9, 16, 17):
-        ranks = np.array([[r + 1 + 12345 + i for i in range(count)] for r in range(nranks)], dtype=np.int32)
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "int32_sum_count32.json")
+    for case in json.load(open(golden))["cases"]:
+        nranks, count = case["team_size"], case["count"]
+        ranks = np.array(case["inputs"], dtype=np.int32)
         src = hip.DeviceBuffer(ranks.nbytes)
         dst = hip.DeviceBuffer(count * 4)
         src.upload(ranks)
         st = rocm.xccl_mem_component_reduce_multi(src.ptr, src.ptr + count * 4, dst.ptr, nranks - 1, count, count * 4,
                                                   Dt.INT32, Op.SUM, MemType.ROCM)
         assert st == Status.OK
-        got = dst.download(np.int32, count)
-        assert got.tolist() == [nranks * (nranks + 1) // 2 + nranks * (i + 12345) for i in range(count)]
+        assert dst.download(np.int32, count).tolist() == case["expected"]
         src.close()
         dst.close()
 

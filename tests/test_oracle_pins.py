@@ -4,6 +4,8 @@ worked out on Python ints, numpy's IEEE arithmetic, and hand-derived truth
 tables.  A dropped term, a swapped operand or a wrong operator column fails at
 least one of these."""
 import itertools
+import json
+import os
 
 import numpy as np
 import pytest
@@ -15,20 +17,25 @@ NP = {0: np.int8, 1: np.int16, 2: np.int32, 3: np.int64, 5: np.uint8, 6: np.uint
       10: np.float16, 11: np.float32, 12: np.float64}
 
 
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "int32_sum_count32.json")
+
+
 def test_reference_known_answer_int32_sum(oracle):
-    """reference test/test_mt.c:58 (same inputs test/test_mpi_allreduce.c:18-21,
-    test/test_mpi_cuda_allreduce.c:35-39): every rank contributes
-    sbuf[i] = rank + 1 + 12345 + i, count 32, INT32 SUM; the result must be
-    P(P+1)/2 + P(i + 12345).  One k-nomial step with radix P is a
-    reduce_multi over P vectors."""
-    count = 32
-    for nranks in range(2, 18):
-        ranks = np.array([[r + 1 + 12345 + i for i in range(count)] for r in range(nranks)], dtype=np.int32)
+    """tests/golden/int32_sum_count32.json = reference test/test_mt.c:58 (same
+    inputs test/test_mpi_allreduce.c:18-21, test/test_mpi_cuda_allreduce.c:35-39):
+    every rank contributes sbuf[i] = rank + 1 + 12345 + i, count 32, INT32 SUM;
+    the result must be P(P+1)/2 + P(i + 12345).  One k-nomial step with radix P
+    is a reduce_multi over P vectors."""
+    cases = json.load(open(GOLDEN))["cases"]
+    assert [c["team_size"] for c in cases] == list(range(2, 18))
+    for c in cases:
+        nranks, count = c["team_size"], c["count"]
+        ranks = np.array(c["inputs"], dtype=np.int32)
         out = np.zeros(count, dtype=np.int32)
         rc = oracle.reduce_multi(ranks, ranks, out, nranks - 1, count, count * 4, Dt.INT32, Op.SUM, off2=count * 4)
         assert rc == 0
-        expect = [nranks * (nranks + 1) // 2 + nranks * (i + 12345) for i in range(count)]
-        assert out.tolist() == expect
+        assert out.tolist() == c["expected"]
+        assert c["expected"] == [nranks * (nranks + 1) // 2 + nranks * (i + 12345) for i in range(count)]
 
 
 @pytest.mark.parametrize("dt", sorted(cmodel.INT_INFO))
