@@ -359,3 +359,33 @@ def test_blocking_calls_from_several_threads(rocm, oracle):
     for c in cases:
         c.close()
     assert not errors, errors
+
+
+def test_blocking_entry_through_graph_path(rocm, oracle):
+    """XCCL_MC_ROCM_GRAPH_MAX_BYTES routes small blocking reductions through the
+    cached single-node graph (read by open()); results must not change, and
+    larger vectors keep the plain launch."""
+    import os
+    vt = rocm.component().super
+    os.environ["XCCL_MC_ROCM_GRAPH_MAX_BYTES"] = "8192"
+    try:
+        assert vt.open() == Status.OK
+        for rep in range(3):
+            for dt, op, size, n2 in ((Dt.FLOAT32, Op.SUM, 2048, 3), (Dt.FLOAT32, Op.SUM, 2049, 3),
+                                     (Dt.INT16, Op.MAX, 4096, 7), (Dt.FLOAT64, Op.PROD, 1000, 1),
+                                     (Dt.UINT8, Op.BOR, 8192, 2), (Dt.INT32, Op.SUM, 1, 15)):
+                c = Case(dt, size, n2)
+                try:
+                    c.fill_random(oracle, 90 + rep, op)
+                    c.upload()
+                    p1, p2, pr = c.ptrs()
+                    assert rocm.xccl_mem_component_reduce_multi(p1, p2, pr, n2, size, c.stride, dt, op,
+                                                                MemType.ROCM) == Status.OK
+                    want, _ = c.expect(oracle, op)
+                    assert_same(c.result(), want, dt, op, "graph-routed %s %s %d" % (Dt(dt).name, Op(op).name, size))
+                finally:
+                    c.close()
+    finally:
+        del os.environ["XCCL_MC_ROCM_GRAPH_MAX_BYTES"]
+        assert vt.open() == Status.OK
+        rocm.component_lib().xccl_rocm_graph_cache_destroy()
