@@ -169,9 +169,11 @@ def main():
               "no inter-GPU work exists to scale) -- use --gpus 1", file=sys.stderr)
         return 2
 
-    from xccl_amd import hip, mc
+    from xccl_amd import build, hip, mc
     from xccl_amd.types import Dt, MemType, Op, Status
 
+    if not build.built():          # load what is built; compile only if nothing is
+        build.build(force=False)
     if hip.device_count() < 1:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 3

@@ -12,6 +12,14 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+@pytest.fixture(scope="session", autouse=True)
+def _native_libraries():
+    """Load what is built; compile only if nothing is (a fresh checkout has no .so files)."""
+    from xccl_amd import build
+    if not build.built():
+        build.build(force=False)
+
+
 def _have_gpu() -> bool:
     try:
         from xccl_amd import hip

@@ -220,10 +220,18 @@ static mc_rocm_event_t *mc_rocm_claim_event(mc_rocm_device_t *d)
     int i, expect;
 
     for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
-        expect = 1;
-        if (atomic_compare_exchange_strong(&d->events[i].is_free, &expect, 0)) {
-            return &d->events[i];
+        mc_rocm_event_t *ev = &d->events[i];
+        expect = MC_SLOT_FREE;
+        if (!atomic_compare_exchange_strong(&ev->is_free, &expect, MC_SLOT_BUSY)) {
+            continue;
         }
+        if (ev->flagged && __atomic_load_n(ev->flag, __ATOMIC_ACQUIRE) != ev->expect) {
+            /* freed by its owner before the launch it stands for finished: its
+             * completion word and arrival counter are still in use */
+            atomic_store(&ev->is_free, MC_SLOT_FREE);
+            continue;
+        }
+        return ev;
     }
     return NULL;
 }
