@@ -129,8 +129,11 @@ typedef struct xccl_rocm_mem_component {
 } xccl_rocm_mem_component_t;
 
 /* Defined by xccl_rocm_mem_component.so; xccl_cuda_mem_component is an alias
- * of the same object. */
-extern xccl_rocm_mem_component_t xccl_rocm_mem_component;
+ * of the same object.  xccl_rocm_mem_component_ext points at it: a loader
+ * that wants the extension looks THAT symbol up, so it never has to read
+ * behind the vtable of a component that may not have one. */
+extern xccl_rocm_mem_component_t        xccl_rocm_mem_component;
+extern xccl_rocm_mem_component_t *const xccl_rocm_mem_component_ext;
 
 /* ------------------------------------------------------------------------
  * Dispatcher (libxccl_mc.so) -- reference src/utils/mem_component.h:52-95,

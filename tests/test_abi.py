@@ -53,6 +53,8 @@ def test_component_object_and_alias():
     for name, _ in mc.MemComponentVtable._fields_[:13]:
         assert ctypes.cast(getattr(vt, name), ctypes.c_void_p).value, "vtable slot %s is NULL" % name
     assert a.ext_version == 1
+    ext = ctypes.c_void_p.in_dll(lib, "xccl_rocm_mem_component_ext")      # how loaders find the extension
+    assert ext.value == ctypes.addressof(a)
     for name in ("reduce_nb", "reduce_multi_nb", "event_wait", "get_stream"):
         assert ctypes.cast(getattr(a, name), ctypes.c_void_p).value
     # 13 function pointers, dlhandle, {buf,size,used(+pad)} on LP64

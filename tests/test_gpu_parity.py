@@ -212,3 +212,24 @@ def test_grid_cap_and_ragged_tiles(rocm, oracle):
             run_and_check(rocm, oracle, dt, op, 1001, 4, off1=dt_size(dt), seed=10)
     finally:
         lib.xccl_rocm_set_launch_shape(0, 1)
+
+
+def test_randomised_shapes(rocm, oracle):
+    """400 reproducible random calls: any supported (dtype, op), 1..20 vectors
+    in sbuf2, sizes up to a few tiles, independent byte placement of the three
+    buffers (element-aligned or not), strides padded by arbitrary byte counts,
+    optionally in place on sbuf1 or sbuf2{0}; each compared with the oracle,
+    bytes outside rbuf included."""
+    rng = np.random.default_rng(20240607)
+    pairs = supported_pairs()
+    for it in range(400):
+        dt, op = pairs[int(rng.integers(len(pairs)))]
+        es = dt_size(dt)
+        n2 = int(rng.integers(1, 21))
+        size = int(rng.choice([1, 2, 3, 15, 16, 17, 63, 64, 65, 127, 129, 1000, 2047, 4097, int(rng.integers(1, 20000))]))
+        unit = es if rng.random() < 0.8 else 1            # mostly element-aligned, sometimes byte-aligned
+        off = [int(rng.integers(0, 64 // unit)) * unit for _ in range(3)]
+        pad = int(rng.integers(0, 5)) * unit * int(rng.choice([0, 1, 3, 16]))
+        alias = [None, None, "s1", ("s2", 0)][int(rng.integers(4))]
+        run_and_check(rocm, oracle, dt, op, size, n2, seed=1000 + it, off1=off[0], off2=off[1], offr=off[2],
+                      stride=size * es + pad, alias=alias)

@@ -21,7 +21,8 @@
 #include <stdlib.h>
 #include <string.h>
 
-static xccl_mem_component_t *mem_components[UCS_MEMORY_TYPE_LAST];
+static xccl_mem_component_t      *mem_components[UCS_MEMORY_TYPE_LAST];
+static xccl_rocm_mem_component_t *mem_extensions[UCS_MEMORY_TYPE_LAST]; /* NULL: plain reference vtable */
 
 /* UCX v1.10 ucs_memory_type_names[], indexed by ucs_memory_type_t */
 static const char *const memory_type_names[UCS_MEMORY_TYPE_LAST] = {
@@ -41,18 +42,10 @@ static xccl_mem_component_t *component_of(int mt)
     return mem_components[mt];
 }
 
-/* The extension, if the component loaded for `mt` is the ROCm one. */
+/* The stream-ordered extension of the component loaded for `mt`, or NULL. */
 static xccl_rocm_mem_component_t *extension_of(int mt)
 {
-    xccl_mem_component_t *mc = component_of(mt);
-
-    if (mc == NULL || (mt != UCS_MEMORY_TYPE_ROCM && mt != UCS_MEMORY_TYPE_ROCM_MANAGED)) {
-        return NULL;
-    }
-    if (((xccl_rocm_mem_component_t *)mc)->ext_version < 1) {
-        return NULL;
-    }
-    return (xccl_rocm_mem_component_t *)mc;
+    return component_of(mt) ? mem_extensions[mt] : NULL;
 }
 
 static xccl_mem_component_t *component_of_stream(xccl_stream_t *stream, int *mt)
@@ -107,6 +100,13 @@ xccl_status_t xccl_mem_component_init(const char *components_path)
         if (mc == NULL || mc->open() != XCCL_OK) {
             dlclose(handle);
             continue;
+        }
+        {
+            /* the extension announces itself through a symbol of its own */
+            xccl_rocm_mem_component_t **ext =
+                (xccl_rocm_mem_component_t **)dlsym(handle, "xccl_rocm_mem_component_ext");
+            mem_extensions[mt] = (ext != NULL && *ext != NULL && &(*ext)->super == mc &&
+                                  (*ext)->ext_version >= 1) ? *ext : NULL;
         }
         mc->dlhandle       = handle;
         mc->cache.size     = cache_size;
@@ -366,6 +366,7 @@ void xccl_mem_component_finalize(void)
         if (mem_components[mt] != NULL) {
             void *handle       = mem_components[mt]->dlhandle;
             mem_components[mt] = NULL;
+            mem_extensions[mt] = NULL;
             dlclose(handle);
         }
     }

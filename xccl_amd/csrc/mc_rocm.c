@@ -626,6 +626,10 @@ xccl_rocm_mem_component_t xccl_rocm_mem_component = {
     .get_stream      = mc_rocm_get_stream,
 };
 
+/* How a loader learns that this component has the extension without reading
+ * past a foreign component's vtable: a second data symbol pointing at it. */
+xccl_rocm_mem_component_t *const xccl_rocm_mem_component_ext = &xccl_rocm_mem_component;
+
 /* The reference loader asks every component file for this one name
  * (src/utils/mem_component.c:30). */
 extern xccl_rocm_mem_component_t xccl_cuda_mem_component
