@@ -62,11 +62,13 @@ xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf,
  * `*dev_flag` -- the device view of a host-mapped 32-bit word -- after its
  * last result store is visible system-wide, and `*flagged` is set to 1; the
  * caller may then poll the host view of the word instead of the stream.
- * `dev_count` is a zeroed 32-bit device word the workgroups count arrivals in;
+ * `dev_count` points at XCCL_ROCM_DONE_COUNT_BYTES of zeroed device memory the
+ * workgroups count arrivals in (two levels, one counter per 128-byte line);
  * the kernel leaves it zero again.  One launch at a time per (count, flag)
  * pair.  For larger launches nothing is attached, `*flagged` is 0 and the
  * caller waits for the stream as usual.  No counterpart in the reference.
  */
+#define XCCL_ROCM_DONE_COUNT_BYTES ((1 + 64) * 128)
 xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbuf,
                                              size_t count, size_t size,
                                              size_t stride, xccl_dt_t dtype,

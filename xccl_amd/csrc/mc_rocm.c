@@ -59,7 +59,7 @@ typedef struct mc_rocm_event {
     uint32_t           expect;    /* last sequence number handed to a kernel */
     volatile uint32_t *flag;      /* host view of the completion word */
     uint32_t          *dev_flag;  /* device view of the same word */
-    uint32_t          *dev_count; /* arrival counter of the launch's workgroups */
+    uint32_t          *dev_count; /* arrival counters of the launch's workgroups */
     hipStream_t        stream;    /* where the work was enqueued */
     unsigned           polls;
 } mc_rocm_event_t;
@@ -138,16 +138,16 @@ static xccl_status_t mc_rocm_device_create(mc_rocm_device_t *d)
                          hipHostMallocMapped));
     memset(d->flag_words, 0, XCCL_ROCM_MC_NUM_EVENTS * MC_FLAG_STRIDE * sizeof(uint32_t));
     MC_HIP(hipMalloc((void **)&d->arrival_counts,
-                     XCCL_ROCM_MC_NUM_EVENTS * sizeof(uint32_t)));
+                     XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_DONE_COUNT_BYTES));
     MC_HIP(hipMemsetAsync(d->arrival_counts, 0,
-                          XCCL_ROCM_MC_NUM_EVENTS * sizeof(uint32_t), d->stream));
+                          XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_DONE_COUNT_BYTES, d->stream));
     MC_HIP(hipStreamSynchronize(d->stream));
     for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
         mc_rocm_event_t *ev = &d->events[i];
         MC_HIP(hipEventCreateWithFlags(&ev->hip_event, hipEventDisableTiming));
         ev->flag = &d->flag_words[i * MC_FLAG_STRIDE];
         MC_HIP(hipHostGetDevicePointer((void **)&ev->dev_flag, (void *)ev->flag, 0));
-        ev->dev_count = &d->arrival_counts[i];
+        ev->dev_count = d->arrival_counts + (size_t)i * (XCCL_ROCM_DONE_COUNT_BYTES / sizeof(uint32_t));
         ev->expect    = 0;
         ev->flagged   = 0;
         atomic_store(&ev->is_free, 1);

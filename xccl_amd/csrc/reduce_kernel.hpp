@@ -38,6 +38,9 @@ constexpr int kBlock = 64; // one wavefront per workgroup
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef u32x4 u32x4_u __attribute__((aligned(1)));
 
+constexpr uint32_t kDoneShards = 64; // second-level arrival counters of a completion word
+constexpr uint32_t kDoneStride = 32; // uint32 words between counters: one per 128-byte line
+
 struct ReduceArgs {
     const char *s1;     // sbuf1
     const char *s2;     // sbuf2 (vector 0)
@@ -50,7 +53,7 @@ struct ReduceArgs {
     // Completion word (small launches only; all NULL/0 otherwise): when the last workgroup
     // is through, done_seq is stored to *done_flag, a host-mapped word the caller polls.
     uint32_t    done_seq;
-    uint32_t   *done_count; // device word, zero between launches
+    uint32_t   *done_count; // device words (1 + kDoneShards, kDoneStride apart), zero between launches
     uint32_t   *done_flag;
 };
 
@@ -249,21 +252,41 @@ __device__ __forceinline__ void fold_tile(const ReduceArgs &a, size_t v0)
 
 // Tells the host that the launch is complete without going through the queue's
 // completion signal (which costs ~4 us more than the kernel's own store on this
-// part).  Every workgroup -- one wave -- first makes its result stores visible
-// system-wide; the last one to arrive publishes the sequence number and re-arms
-// the arrival counter.  One contended atomic per workgroup: for small grids only.
-__device__ __forceinline__ void publish_completion(const ReduceArgs &a)
+// part).  Every workgroup -- one wave -- waits until its own result stores have
+// completed, then counts itself in; the last one to arrive publishes the
+// sequence number and re-arms the counter.
+//   Streaming policy: the vector stores are system-scope write-through, so
+//   "completed" already means "in memory"; a wave only needs its vmcnt to
+//   drain (a workgroup-scope release) before it counts itself in.  Stores made
+//   with default policy (`wrote_plain`: the element-wise head/tail, or every
+//   store under POL_PLAIN) sit dirty in this XCD's L2 and need the wave's own
+//   system-scope release, which writes that L2 back.
+// One contended atomic per workgroup: for small grids only.
+template <int POL>
+__device__ __forceinline__ void publish_completion(const ReduceArgs &a, bool wrote_plain)
 {
-    __threadfence_system();
+    if (POL != POL_STREAM || wrote_plain) {
+        __threadfence_system();
+    } else {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    }
     if (threadIdx.x == 0) {
-        bool last = true;
-        if (gridDim.x > 1) {
-            const uint32_t before =
-                __hip_atomic_fetch_add(a.done_count, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-            last = before == gridDim.x - 1;
-            if (last) {
-                __hip_atomic_store(a.done_count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+        // Arrival counting in two levels, so that no single word takes more than
+        // grid/kDoneShards increments: workgroup b counts into shard b % shards, the
+        // wave that fills a shard counts into word 0, the wave that fills word 0 is
+        // the last.  atomicInc wraps to zero at its bound, so every word is back at
+        // zero by itself when the launch is over.  Words are kDoneStride apart
+        // (one per 128-byte line): [0] top, [1 + s] shard s.
+        const uint32_t grid   = gridDim.x;
+        const uint32_t shards = grid < kDoneShards ? grid : kDoneShards;
+        bool           last   = true;
+        if (grid > kDoneShards) {
+            const uint32_t sh    = blockIdx.x % kDoneShards;
+            const uint32_t total = grid / kDoneShards + (sh < grid % kDoneShards ? 1u : 0u);
+            last = atomicInc(a.done_count + (1 + sh) * kDoneStride, total - 1) == total - 1;
+        }
+        if (last && grid > 1) {
+            last = atomicInc(a.done_count, shards - 1) == shards - 1;
         }
         if (last) {
             __hip_atomic_store(a.done_flag, a.done_seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -283,7 +306,8 @@ __global__ void __launch_bounds__(kBlock) reduce_multi_kernel(const ReduceArgs a
             fold_tile<T, Op, NSRC, UNROLL, POL, true>(a, v0);
         }
     }
-    if (blockIdx.x == gridDim.x - 1) {
+    const bool edges = blockIdx.x == gridDim.x - 1 && a.head + a.tail != 0;
+    if (edges) {
         const size_t t = threadIdx.x;
         if (t < a.head) {
             fold_element<T, Op>(a, t);
@@ -292,7 +316,7 @@ __global__ void __launch_bounds__(kBlock) reduce_multi_kernel(const ReduceArgs a
         }
     }
     if (a.done_flag != nullptr) {
-        publish_completion(a);
+        publish_completion<POL>(a, edges);
     }
 }
 

@@ -204,9 +204,11 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
 }
 
 // Launches of at most this many workgroups may carry a completion word: each
-// workgroup pays one atomic on a shared counter, which is nothing for a few
-// hundred and would serialise a grid of hundreds of thousands.
-constexpr unsigned kMaxFlaggedGrid = 512;
+// workgroup pays an atomic on one of 64 shared counters (~12 ns per arrival
+// on the same word, measured), which beats the queue's completion signal up
+// to here and would serialise a grid of hundreds of thousands.
+constexpr unsigned kMaxFlaggedGrid = 8192;
+static_assert(XCCL_ROCM_DONE_COUNT_BYTES == (1 + kDoneShards) * kDoneStride * sizeof(uint32_t), "counter block size");
 
 // ---- single-kernel-node graph cache ---------------------------------------
 constexpr int kGraphSlots = 8;
