@@ -76,8 +76,9 @@ typedef struct mc_rocm_stream_request {
 
 typedef struct mc_rocm_device {
     atomic_int               ready; /* 0 = untouched, 1 = usable */
-    hipStream_t              stream;
-    int                     *gate_words; /* pinned, mapped */
+    hipStream_t              stream;      /* reductions */
+    hipStream_t              gate_stream; /* stream gates: a gate must never sit in front of a reduction */
+    int                     *gate_words;  /* pinned, mapped */
     uint32_t                *flag_words; /* pinned, mapped: completion words of the events */
     uint32_t                *arrival_counts; /* device */
     mc_rocm_event_t          events[XCCL_ROCM_MC_NUM_EVENTS];
@@ -123,6 +124,7 @@ static xccl_status_t mc_rocm_device_create(mc_rocm_device_t *d)
     int i;
 
     MC_HIP(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
+    MC_HIP(hipStreamCreateWithFlags(&d->gate_stream, hipStreamNonBlocking));
     MC_HIP(hipHostMalloc((void **)&d->gate_words,
                          XCCL_ROCM_MC_NUM_STREAM_REQUESTS * sizeof(int),
                          hipHostMallocMapped));
@@ -490,8 +492,11 @@ static xccl_status_t mc_rocm_event_free(xccl_mc_event_t *event)
 }
 
 /* cuda_mem_component.c:139-162: block the USER's stream until the host calls
- * finish_stream_activity.  A gate kernel on the component stream polls a
- * host-mapped word; the user stream waits on an event recorded behind it. */
+ * finish_stream_activity.  A gate kernel polls a host-mapped word; the user
+ * stream waits on an event recorded behind it.  Gates run on a stream of their
+ * own: the reference puts its spin kernel on the stream its reductions use,
+ * so a reduction issued while a gate is shut would wait for the very
+ * collective that is waiting for the reduction. */
 static xccl_status_t
 mc_rocm_start_stream_activity(xccl_stream_t *stream,
                               xccl_mem_component_stream_request_t **req)
@@ -526,12 +531,12 @@ mc_rocm_start_stream_activity(xccl_stream_t *stream,
         return XCCL_ERR_NO_RESOURCE;
     }
     __atomic_store_n(r->flag, 0, __ATOMIC_RELEASE);
-    st = xccl_rocm_stream_gate(r->dev_flag, mc_gate_timeout_ns, d->stream);
+    st = xccl_rocm_stream_gate(r->dev_flag, mc_gate_timeout_ns, d->gate_stream);
     if (st != XCCL_OK) {
         atomic_store(&r->is_free, 1);
         return st;
     }
-    if (hipEventRecord(r->hip_event, d->stream) != hipSuccess ||
+    if (hipEventRecord(r->hip_event, d->gate_stream) != hipSuccess ||
         hipStreamWaitEvent(user, r->hip_event, 0) != hipSuccess) {
         /* open the gate again: nothing may stay blocked behind a failure */
         __atomic_store_n(r->flag, 1, __ATOMIC_RELEASE);
@@ -586,6 +591,10 @@ static void mc_rocm_close(void)
     d = &mc_devices[dev];
     pthread_mutex_lock(&mc_init_lock);
     if (atomic_load(&d->ready) == 1) {
+        for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS; i++) {
+            __atomic_store_n(d->requests[i].flag, 1, __ATOMIC_RELEASE); /* open any gate left shut */
+        }
+        (void)hipStreamSynchronize(d->gate_stream);
         (void)hipStreamSynchronize(d->stream);
         xccl_rocm_graph_cache_destroy();
         for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
@@ -597,6 +606,7 @@ static void mc_rocm_close(void)
         (void)hipHostFree(d->gate_words);
         (void)hipHostFree(d->flag_words);
         (void)hipFree(d->arrival_counts);
+        (void)hipStreamDestroy(d->gate_stream);
         (void)hipStreamDestroy(d->stream);
         memset(d, 0, sizeof(*d));
     }
