@@ -401,3 +401,49 @@ def test_blocking_entry_through_graph_path(rocm, oracle):
         del os.environ["XCCL_MC_ROCM_GRAPH_MAX_BYTES"]
         assert vt.open() == Status.OK
         rocm.component_lib().xccl_rocm_graph_cache_destroy()
+
+
+def test_stream_ordered_entries_under_stream_capture(rocm, oracle):
+    """A caller records a whole k-nomial step sequence -- three dependent
+    reduce_multi_nb launches on its own stream, no events -- into a hipGraph
+    and replays it.  Every replay, with eager work and synchronisation in
+    between, must reproduce the eager result (the entries enqueue kernels only:
+    no memset nodes, no allocation)."""
+    dt, op, size, n2 = Dt.FLOAT32, Op.SUM, 50000, 3
+    c = Case(dt, size, n2)
+    s = rocm.Stream(hip.stream_create())
+    try:
+        c.fill_random(oracle, 33)
+        c.upload()
+        p1, p2, pr = c.ptrs()
+
+        def enqueue():
+            for first in (p1, pr, pr):     # round 1 reads sbuf1, later rounds run in place on rbuf
+                st, ev = rocm.xccl_mem_component_reduce_multi_nb(first, p2, pr, n2, size, c.stride, dt, op,
+                                                                 MemType.ROCM, s, want_event=False)
+                assert st == Status.OK and not ev
+
+        enqueue()
+        hip.stream_synchronize(s.hip_stream)
+        eager = c.result().copy()
+        img = c.host.copy()
+        b = img.ctypes.data
+        for first in (c.o1, c.orr, c.orr):
+            oracle.reduce_multi_ptr(b + first, b + c.o2, b + c.orr, n2, size, c.stride, dt, op)
+        assert_same(eager, img[c.orr: c.orr + c.vbytes], dt, op, "eager chain")
+
+        hip.stream_begin_capture(s.hip_stream)
+        enqueue()
+        graph = hip.stream_end_capture(s.hip_stream)
+        gexec = hip.graph_instantiate(graph)
+        for rep in range(4):
+            hip.memset(pr, 0x3C, c.vbytes)
+            hip.graph_launch(gexec, s.hip_stream)
+            hip.stream_synchronize(s.hip_stream)
+            assert_same(c.result(), eager, dt, op, "graph replay %d" % rep)
+            # eager work of the component between replays
+            assert rocm.xccl_mem_component_reduce(p1, p2, pr, size, dt, op, MemType.ROCM) == Status.OK
+        hip.graph_destroy(graph, gexec)
+    finally:
+        c.close()
+        hip.stream_destroy(s.hip_stream)

@@ -185,3 +185,32 @@ class DeviceBuffer:
             self.close()
         except Exception:
             pass
+
+
+# ---- stream capture / graphs (for callers that record the component's launches into their own graph) ----
+
+def stream_begin_capture(s: int, mode: int = 0):
+    check(lib().hipStreamBeginCapture(ctypes.c_void_p(s), ctypes.c_int(mode)), "hipStreamBeginCapture")
+
+
+def stream_end_capture(s: int) -> int:
+    g = ctypes.c_void_p()
+    check(lib().hipStreamEndCapture(ctypes.c_void_p(s), ctypes.byref(g)), "hipStreamEndCapture")
+    return g.value
+
+
+def graph_instantiate(graph: int) -> int:
+    e = ctypes.c_void_p()
+    check(lib().hipGraphInstantiate(ctypes.byref(e), ctypes.c_void_p(graph), None, None, ctypes.c_size_t(0)),
+          "hipGraphInstantiate")
+    return e.value
+
+
+def graph_launch(graph_exec: int, s: int):
+    check(lib().hipGraphLaunch(ctypes.c_void_p(graph_exec), ctypes.c_void_p(s)), "hipGraphLaunch")
+
+
+def graph_destroy(graph: int, graph_exec: int = 0):
+    if graph_exec:
+        check(lib().hipGraphExecDestroy(ctypes.c_void_p(graph_exec)), "hipGraphExecDestroy")
+    check(lib().hipGraphDestroy(ctypes.c_void_p(graph)), "hipGraphDestroy")
