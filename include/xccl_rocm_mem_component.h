@@ -108,6 +108,10 @@ extern "C" {
  *                    XCCL_OK), block on it with event_wait, return it with
  *                    event_free.  XCCL_ERR_NO_RESOURCE when the pool is empty
  *                    (nothing is enqueued then).
+ * With event == NULL the entries do nothing but enqueue one kernel, so a
+ * caller may record them into its own hipGraph through stream capture; an
+ * event must not be requested while capturing (its completion is tied to
+ * this one launch, not to later replays).
  * These replace the launch + cudaStreamSynchronize pair of the reference
  * (xccl_cuda_reduce_multi.cu:42-44,140) at the call sites named above.
  */

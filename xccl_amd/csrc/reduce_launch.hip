@@ -358,20 +358,8 @@ xccl_status_t xccl_rocm_reduce_supported(xccl_dt_t dtype, xccl_op_t op)
 xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
                                           size_t stride, xccl_dt_t dtype, xccl_op_t op, void *hip_stream)
 {
-    if (lookup(dtype, op) == nullptr) {
-        return XCCL_ERR_UNSUPPORTED;
-    }
-    if (size == 0) {
-        return XCCL_OK;
-    }
-    Plan          plan;
-    xccl_status_t st = make_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan);
-    if (st != XCCL_OK) {
-        return st;
-    }
-    void *argv[1] = {&plan.args};
-    HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, 0, (hipStream_t)hip_stream));
-    return XCCL_OK;
+    return xccl_rocm_reduce_multi_flagged(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, hip_stream, nullptr,
+                                          nullptr, 0, nullptr);
 }
 
 xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
