@@ -206,3 +206,17 @@ def test_large_vectors_stream_ordered_overlap(rocm, oracle):
             assert np.array_equal(rk.result(r), want)
         assert stats["reduce_inflight_returns"] > 0
         rk.close()
+
+
+def test_c_program_in_the_shape_of_the_reference_tests():
+    """tests/c/test_rocm_allreduce.c: a C program laid out like
+    test/test_mpi_cuda_allreduce.c and test/test_mpi_cuda_reduce.c, driving the
+    dispatcher and the component from C only (built by xccl_amd/csrc/Makefile)."""
+    import os
+    import subprocess
+    from xccl_amd.build import LIB_DIR
+    exe = os.path.join(LIB_DIR, "test_rocm_allreduce")
+    for team, count in ((8, 32), (6, 32), (17, 32), (5, 100000)):
+        out = subprocess.run([exe, LIB_DIR, str(team), str(count)], capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stdout + out.stderr
+        assert "Correctness check: PASSED" in out.stdout

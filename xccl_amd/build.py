@@ -6,7 +6,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 
-LIBS = ("xccl_rocm_mem_component.so", "libxccl_mc.so", "libxccl_rocm_benchkit.so", "libxccl_ucx_replay.so")
+LIBS = ("xccl_rocm_mem_component.so", "libxccl_mc.so", "libxccl_rocm_benchkit.so", "libxccl_ucx_replay.so",
+        "test_rocm_allreduce")
 
 
 def built() -> bool:
