@@ -97,11 +97,16 @@ void xccl_rocm_graph_cache_destroy(void);
  * workgroups loop over tiles.  0 restores the built-in default (a cap large
  * enough that every tile gets its own workgroup).  `cache_policy`: 1 =
  * streaming accesses (non-temporal loads, system-scope stores; the default),
- * 0 = default-policy loads and stores.  Both are process-global and may also
- * be set through the environment (XCCL_MC_ROCM_BLOCKS_PER_CU,
- * XCCL_MC_ROCM_CACHE_POLICY), read once at first launch.
+ * 0 = default-policy loads and stores.  `resident_per_cu`: how many
+ * workgroups may be resident on a compute unit at once (enforced by asking
+ * for LDS the kernel never touches); 0 = the built-in choice by source count
+ * (8 to 12), 32 or more = no limit.  All are process-global and may also be
+ * set through the environment (XCCL_MC_ROCM_BLOCKS_PER_CU,
+ * XCCL_MC_ROCM_CACHE_POLICY, XCCL_MC_ROCM_RESIDENT_PER_CU), read once at
+ * first launch.
  */
-void xccl_rocm_set_launch_shape(int blocks_per_cu, int cache_policy);
+void xccl_rocm_set_launch_shape(int blocks_per_cu, int cache_policy,
+                                int resident_per_cu);
 
 /* What a launch with these arguments would be: grid/block size and the
  * mangled kernel name (truncated into `name`, if not NULL).  Host-only apart

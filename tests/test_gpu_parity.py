@@ -202,16 +202,16 @@ def test_grid_cap_and_ragged_tiles(rocm, oracle):
     lib = rocm.component_lib()
     try:
         for bpc in (1, 64):
-            lib.xccl_rocm_set_launch_shape(bpc, 1)
+            lib.xccl_rocm_set_launch_shape(bpc, 1, 0)
             for size in (256 * 4 * 2 * 256 + 13, 1 << 20, (1 << 20) + 4 * 255 + 3):
                 run_and_check(rocm, oracle, Dt.FLOAT32, Op.SUM, size, 7, seed=9, check_untouched=False)
                 run_and_check(rocm, oracle, Dt.INT8, Op.SUM, size, 2, seed=9, check_untouched=False)
-        lib.xccl_rocm_set_launch_shape(0, 0)   # default-policy loads and stores instead of streaming ones
+        lib.xccl_rocm_set_launch_shape(0, 0, 32)   # default-policy loads and stores, no residency cap
         for dt, op in ((Dt.FLOAT32, Op.SUM), (Dt.INT16, Op.MAX), (Dt.FLOAT64, Op.MIN)):
             run_and_check(rocm, oracle, dt, op, (1 << 18) + 77, 7, seed=10)
             run_and_check(rocm, oracle, dt, op, 1001, 4, off1=dt_size(dt), seed=10)
     finally:
-        lib.xccl_rocm_set_launch_shape(0, 1)
+        lib.xccl_rocm_set_launch_shape(0, 1, 0)
 
 
 def test_randomised_shapes(rocm, oracle):

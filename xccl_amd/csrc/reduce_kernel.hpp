@@ -14,7 +14,11 @@
 // workgroups, one tile per workgroup (a grid as large as the tile count; the
 // grid-stride loop only runs when that exceeds the grid cap) beat 256-lane
 // persistent workgroups by ~25%; streaming cache policy (non-temporal loads,
-// system-scope write-through stores) beats default-policy accesses by ~17%.
+// system-scope write-through stores) beats default-policy accesses by ~17%;
+// holding the workgroups resident per compute unit to about ten (the launch
+// asks for LDS it never touches) adds 4-12%: the memory side is saturated
+// long before the wave slots are, and fewer waves in flight keep the
+// addresses being served close together.
 //
 // Layout of one call, in elements of T:
 //     [0, head)                 peeled so that the vector body starts on a
@@ -42,9 +46,9 @@ constexpr uint32_t kDoneShards = 64; // second-level arrival counters of a compl
 constexpr uint32_t kDoneStride = 32; // uint32 words between counters: one per 128-byte line
 
 struct ReduceArgs {
-    const char *s1;     // sbuf1
-    const char *s2;     // sbuf2 (vector 0)
-    char       *dst;    // rbuf / target
+    const char *s1;     // sbuf1, at the first byte of the vector body (head elements lie before it)
+    const char *s2;     // sbuf2 (vector 0), likewise
+    char       *dst;    // rbuf / target, likewise
     size_t      stride; // bytes between vectors of sbuf2
     size_t      head;   // elements before the vector body
     size_t      nvec;   // 16-byte vectors in the body
@@ -112,29 +116,39 @@ template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBxor>(u32x4 a, u32
 //               i.e. write through instead of lingering dirty in L2.
 enum { POL_PLAIN = 0, POL_STREAM = 1 };
 
+// Vector accesses are addressed as (uniform 64-bit base) + (32-bit lane
+// offset): the base lives in scalar registers, one VGPR serves every access of
+// a tile, and a wave gets from its first instruction to its first load in a
+// few cycles -- with one tile per wave, the prologue is part of every tile.
 template <int POL>
-__device__ __forceinline__ u32x4 vload(const char *p)
+__device__ __forceinline__ u32x4 vload(const char *base, uint32_t off)
 {
     if (POL == POL_STREAM) {
-        return __builtin_nontemporal_load((const u32x4_u *)p);
+        return __builtin_nontemporal_load((const u32x4_u *)(base + off));
     }
-    return *(const u32x4_u *)p;
+    return *(const u32x4_u *)(base + off);
 }
 
 template <int POL>
-__device__ __forceinline__ void vstore(char *p, u32x4 v)
+__device__ __forceinline__ void vstore(char *base, uint32_t off, u32x4 v)
 {
     if (POL == POL_STREAM) {
-        // No builtin emits a 16-byte store with these scope bits, hence asm.
+        // No builtin emits a 16-byte store with these scope bits, hence asm --
+        // and asm the compiler's hazard recogniser cannot see into, so the
+        // statement has to be hazard-free by construction:
+        //  * it takes its address as a 64-bit VGPR pair, never a scalar base:
+        //    a VMEM instruction that reads an SGPR within 5 wait states of a
+        //    VALU write to it (v_readlane restoring a spilled SGPR does that)
+        //    sees the old value, i.e. a wild address;
+        //  * it ends in s_nop: gfx9 reads the data registers of a store wider
+        //    than 8 bytes one cycle after issue, and a VALU write to them in
+        //    the next slot corrupts the stored value.
         // A store has no result register, so the compiler's s_waitcnt
-        // bookkeeping stays valid; the clobber keeps it ordered after the
-        // loads.  The s_nop is required: gfx9 reads the data registers of a
-        // store wider than 8 bytes one cycle after issue, and a VALU write to
-        // them in the very next slot corrupts the stored value.  The compiler
-        // pads that hazard for its own stores but cannot see into the asm.
+        // bookkeeping stays valid; the clobber keeps it ordered after the loads.
+        char *p = base + off;
         asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
     } else {
-        *(u32x4_u *)p = v;
+        *(u32x4_u *)(base + off) = v;
     }
 }
 
@@ -146,16 +160,16 @@ __device__ __forceinline__ T eload(const char *p)
     return v;
 }
 
-// One element, all sources, in fold order.
+// One element, all sources, in fold order.  `rel`: byte offset of the element
+// from the start of the vector body (negative in the head).
 template <typename T, class Op>
-__device__ __forceinline__ void fold_element(const ReduceArgs &a, size_t e)
+__device__ __forceinline__ void fold_element(const ReduceArgs &a, ptrdiff_t rel)
 {
-    const size_t off = e * sizeof(T);
-    T acc = Op::template f<T>(eload<T>(a.s1 + off), eload<T>(a.s2 + off));
+    T acc = Op::template f<T>(eload<T>(a.s1 + rel), eload<T>(a.s2 + rel));
     for (uint32_t j = 1; j < a.n2; ++j) {
-        acc = Op::template f<T>(eload<T>(a.s2 + (size_t)j * a.stride + off), acc);
+        acc = Op::template f<T>(eload<T>(a.s2 + (size_t)j * a.stride + rel), acc);
     }
-    __builtin_memcpy(a.dst + off, &acc, sizeof(T));
+    __builtin_memcpy(a.dst + rel, &acc, sizeof(T));
 }
 
 // One tile = UNROLL x kBlock vectors; lane t of the block owns vectors
@@ -165,14 +179,16 @@ __device__ __forceinline__ void fold_element(const ReduceArgs &a, size_t e)
 template <typename T, class Op, int NSRC, int UNROLL, int POL, bool GUARD>
 __device__ __forceinline__ void fold_tile(const ReduceArgs &a, size_t v0)
 {
-    const size_t body = a.head * sizeof(T);
-    size_t       off[UNROLL];
+    const size_t tile_off = v0 * 16; // uniform: same for every lane of the workgroup
+    const char  *p1       = a.s1 + tile_off;
+    const char  *p2       = a.s2 + tile_off;
+    char        *pd       = a.dst + tile_off;
+    uint32_t     off[UNROLL];
     bool         live[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-        const size_t v = v0 + (size_t)u * kBlock + threadIdx.x;
-        live[u]        = !GUARD || v < a.nvec;
-        off[u]         = body + v * 16;
+        off[u]  = (uint32_t)(u * kBlock + (int)threadIdx.x) * 16u;
+        live[u] = !GUARD || v0 + (size_t)u * kBlock + threadIdx.x < a.nvec;
     }
 
     if constexpr (NSRC > 0) {
@@ -181,10 +197,10 @@ __device__ __forceinline__ void fold_tile(const ReduceArgs &a, size_t v0)
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             if (live[u]) {
-                r[u][0] = vload<POL>(a.s1 + off[u]);
+                r[u][0] = vload<POL>(p1, off[u]);
 #pragma unroll
                 for (int j = 1; j < N; ++j) {
-                    r[u][j] = vload<POL>(a.s2 + (size_t)(j - 1) * a.stride + off[u]);
+                    r[u][j] = vload<POL>(p2 + (size_t)(j - 1) * a.stride, off[u]);
                 }
             }
         }
@@ -196,7 +212,7 @@ __device__ __forceinline__ void fold_tile(const ReduceArgs &a, size_t v0)
                 for (int j = 2; j < N; ++j) {
                     acc = vfold<T, Op>(r[u][j], acc);
                 }
-                vstore<POL>(a.dst + off[u], acc);
+                vstore<POL>(pd, off[u], acc);
             }
         }
     } else {
@@ -204,21 +220,21 @@ __device__ __forceinline__ void fold_tile(const ReduceArgs &a, size_t v0)
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             if (live[u]) {
-                u32x4 x = vload<POL>(a.s1 + off[u]);
-                u32x4 y = vload<POL>(a.s2 + off[u]);
+                u32x4 x = vload<POL>(p1, off[u]);
+                u32x4 y = vload<POL>(p2, off[u]);
                 acc[u]  = vfold<T, Op>(x, y);
             }
         }
         uint32_t j = 1;
         for (; j + 4 <= a.n2; j += 4) {
-            const char *p = a.s2 + (size_t)j * a.stride;
+            const char *p = p2 + (size_t)j * a.stride;
             u32x4       r[UNROLL][4];
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 if (live[u]) {
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
-                        r[u][k] = vload<POL>(p + (size_t)k * a.stride + off[u]);
+                        r[u][k] = vload<POL>(p + (size_t)k * a.stride, off[u]);
                     }
                 }
             }
@@ -233,18 +249,18 @@ __device__ __forceinline__ void fold_tile(const ReduceArgs &a, size_t v0)
             }
         }
         for (; j < a.n2; ++j) {
-            const char *p = a.s2 + (size_t)j * a.stride;
+            const char *p = p2 + (size_t)j * a.stride;
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 if (live[u]) {
-                    acc[u] = vfold<T, Op>(vload<POL>(p + off[u]), acc[u]);
+                    acc[u] = vfold<T, Op>(vload<POL>(p, off[u]), acc[u]);
                 }
             }
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             if (live[u]) {
-                vstore<POL>(a.dst + off[u], acc[u]);
+                vstore<POL>(pd, off[u], acc[u]);
             }
         }
     }
@@ -299,23 +315,48 @@ __global__ void __launch_bounds__(kBlock) reduce_multi_kernel(const ReduceArgs a
 {
     constexpr size_t tile = (size_t)kBlock * UNROLL;
     const size_t     step = (size_t)gridDim.x * tile;
-    for (size_t v0 = (size_t)blockIdx.x * tile; v0 < a.nvec; v0 += step) {
-        if (v0 + tile <= a.nvec) {
-            fold_tile<T, Op, NSRC, UNROLL, POL, false>(a, v0);
-        } else {
-            fold_tile<T, Op, NSRC, UNROLL, POL, true>(a, v0);
-        }
-    }
+    size_t           v0   = (size_t)blockIdx.x * tile;
+
+    // Fetch the completion-word pointer together with the other arguments: left
+    // alone, its scalar load sinks below the stores and the wave waits for it
+    // there instead of retiring.
+    uint32_t *const done_flag = a.done_flag;
+    asm volatile("" : : "s"(done_flag));
+
+    // Head and tail first: they use ordinary loads and stores, whose completion
+    // the compiler tracks.  The tiles end in asm stores it cannot see; anything
+    // it had to order after them (a loop back-edge, say) would make it wait for
+    // every outstanding store, and the wave would sit on its slot for a
+    // write-through round trip instead of retiring.
     const bool edges = blockIdx.x == gridDim.x - 1 && a.head + a.tail != 0;
     if (edges) {
         const size_t t = threadIdx.x;
         if (t < a.head) {
-            fold_element<T, Op>(a, t);
+            fold_element<T, Op>(a, -(ptrdiff_t)((a.head - t) * sizeof(T)));
         } else if (t - a.head < a.tail) {
-            fold_element<T, Op>(a, a.head + a.nvec * Vec<T>::n + (t - a.head));
+            fold_element<T, Op>(a, (ptrdiff_t)(a.nvec * 16 + (t - a.head) * sizeof(T)));
         }
     }
-    if (a.done_flag != nullptr) {
+    if (step >= a.nvec) {
+        // the usual launch: at most one tile per workgroup, straight-line code
+        if (v0 < a.nvec) {
+            if (v0 + tile <= a.nvec) {
+                fold_tile<T, Op, NSRC, UNROLL, POL, false>(a, v0);
+            } else {
+                fold_tile<T, Op, NSRC, UNROLL, POL, true>(a, v0);
+            }
+        }
+    } else {
+        // more tiles than the grid cap allows workgroups: loop
+        for (; v0 < a.nvec; v0 += step) {
+            if (v0 + tile <= a.nvec) {
+                fold_tile<T, Op, NSRC, UNROLL, POL, false>(a, v0);
+            } else {
+                fold_tile<T, Op, NSRC, UNROLL, POL, true>(a, v0);
+            }
+        }
+    }
+    if (done_flag != nullptr) {
         publish_completion<POL>(a, edges);
     }
 }
@@ -326,8 +367,11 @@ __global__ void __launch_bounds__(kBlock) reduce_multi_kernel(const ReduceArgs a
 enum { NV_ANY = 0, NV_2, NV_3, NV_4, NV_8, NV_16, NV_COUNT };
 
 constexpr int nsrc_of(int nv) { return nv == NV_2 ? 2 : nv == NV_3 ? 3 : nv == NV_4 ? 4 : nv == NV_8 ? 8 : nv == NV_16 ? 16 : 0; }
-// vectors per lane per tile (measured: more than ~8 loads in flight per lane buys nothing)
-constexpr int unroll_of(int nv) { return nv == NV_2 ? 2 : nv == NV_3 ? 2 : nv == NV_4 ? 2 : nv == NV_8 ? 1 : nv == NV_16 ? 1 : 2; }
+// vectors per lane per tile: two -- with the resident-workgroup cap, two tiles
+// per wave measured best for 2, 4, 8 and 16 sources alike -- except 16 sources
+// of 8-bit elements, where 32 vectors in flight plus the unpacked bytes do not
+// fit the register file and the compiler would spill to scratch memory
+constexpr int unroll_of(int nv, int esize) { return (nv == NV_16 && esize == 1) ? 1 : 2; }
 
 struct KernelEntry {
     const void *fn[2][NV_COUNT]; // [cache policy][variant]
@@ -337,7 +381,7 @@ struct KernelEntry {
 template <typename T, class Op, int POL, int NV>
 constexpr const void *kernel_ptr()
 {
-    return (const void *)&reduce_multi_kernel<T, Op, nsrc_of(NV), unroll_of(NV), POL>;
+    return (const void *)&reduce_multi_kernel<T, Op, nsrc_of(NV), unroll_of(NV, (int)sizeof(T)), POL>;
 }
 
 template <typename T, class Op>

@@ -18,8 +18,15 @@ constexpr int kMaxDevices       = 64;
 // workgroup measured fastest, so the cap only bounds the grid of huge calls.
 constexpr int kDefaultBlocksPerCu = 8192;
 
+// Resident one-wave workgroups per compute unit for large launches, by source
+// count (0 = these defaults, > 0 = this many for every call, >= kNoResidentCap =
+// no cap).  Measured optimum on MI355X: 12 for 2-3 sources, 10 up to 8, 8 beyond.
+constexpr int    kNoResidentCap = 32;
+constexpr size_t kLdsPerCu      = 160 * 1024;
+
 std::atomic<int> g_blocks_per_cu{-1}; // -1: not read from the environment yet
 std::atomic<int> g_policy{-1};
+std::atomic<int> g_resident{0};
 std::atomic<int> g_cu_count[kMaxDevices];
 
 void read_env_once()
@@ -29,7 +36,9 @@ void read_env_once()
     }
     const char *pol = getenv("XCCL_MC_ROCM_CACHE_POLICY");
     const char *bpc = getenv("XCCL_MC_ROCM_BLOCKS_PER_CU");
+    const char *res = getenv("XCCL_MC_ROCM_RESIDENT_PER_CU");
     int         v   = bpc ? atoi(bpc) : 0;
+    g_resident.store(res && atoi(res) > 0 ? atoi(res) : 0, std::memory_order_release);
     g_policy.store((pol && atoi(pol) == POL_PLAIN) ? POL_PLAIN : POL_STREAM, std::memory_order_release);
     g_blocks_per_cu.store(v > 0 ? v : kDefaultBlocksPerCu, std::memory_order_release);
 }
@@ -111,12 +120,26 @@ const KernelEntry *lookup(xccl_dt_t dt, xccl_op_t op)
 struct Plan {
     const void *fn;
     unsigned    grid;
+    unsigned    lds_bytes; // dynamic LDS asked for only to bound resident workgroups per CU
     ReduceArgs  args;
 };
 
+// LDS per workgroup that lets `resident` workgroups share a compute unit.
+unsigned lds_for_resident(uint32_t nsrc, size_t grid, int cus)
+{
+    int cap = g_resident.load(std::memory_order_relaxed);
+    if (cap == 0) {
+        cap = nsrc <= 3 ? 12 : nsrc <= 8 ? 10 : 8;
+    }
+    if (cap >= kNoResidentCap || grid <= (size_t)cap * (size_t)cus) {
+        return 0; // the whole grid is resident at once anyway
+    }
+    return (unsigned)((kLdsPerCu / (size_t)cap) & ~(size_t)511);
+}
+
 bool same_plan(const Plan &a, const Plan &b)
 {
-    return a.fn == b.fn && a.grid == b.grid && a.args.s1 == b.args.s1 && a.args.s2 == b.args.s2 &&
+    return a.fn == b.fn && a.grid == b.grid && a.lds_bytes == b.lds_bytes && a.args.s1 == b.args.s1 && a.args.s2 == b.args.s2 &&
            a.args.dst == b.args.dst && a.args.stride == b.args.stride && a.args.head == b.args.head &&
            a.args.nvec == b.args.nvec && a.args.tail == b.args.tail && a.args.n2 == b.args.n2 &&
            a.args.done_flag == b.args.done_flag && a.args.done_seq == b.args.done_seq;
@@ -179,9 +202,9 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
         head = elems;
     }
     ReduceArgs &a = plan->args;
-    a.s1     = (const char *)s1;
-    a.s2     = (const char *)s2;
-    a.dst    = (char *)dst;
+    a.s1     = (const char *)s1 + head * esize; // the kernel works relative to the vector body
+    a.s2     = (const char *)s2 + head * esize;
+    a.dst    = (char *)dst + head * esize;
     a.stride = stride;
     a.head   = head;
     a.nvec   = (elems - head) / ve;
@@ -191,14 +214,15 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     a.done_count = nullptr;
     a.done_flag  = nullptr;
 
-    const size_t tile  = (size_t)kBlock * unroll_of(nv);
+    const size_t tile  = (size_t)kBlock * unroll_of(nv, e->elem_size);
     const size_t tiles = (a.nvec + tile - 1) / tile;
     const size_t cap   = (size_t)cus * (size_t)g_blocks_per_cu.load(std::memory_order_relaxed);
     size_t       grid  = tiles < cap ? tiles : cap;
     if (grid == 0) {
         grid = 1; // head/tail only
     }
-    plan->grid = (unsigned)grid;
+    plan->grid      = (unsigned)grid;
+    plan->lds_bytes = lds_for_resident(nsrc, grid, cus);
     plan->fn   = e->fn[g_policy.load(std::memory_order_relaxed) == POL_PLAIN ? POL_PLAIN : POL_STREAM][nv];
     return XCCL_OK;
 }
@@ -238,7 +262,7 @@ void fill_node_params(hipKernelNodeParams *p, Plan *plan, void **argv)
     p->func           = const_cast<void *>(plan->fn);
     p->gridDim        = dim3(plan->grid, 1, 1);
     p->blockDim       = dim3(kBlock, 1, 1);
-    p->sharedMemBytes = 0;
+    p->sharedMemBytes = plan->lds_bytes;
     p->kernelParams   = argv;
     p->extra          = nullptr;
 }
@@ -387,7 +411,8 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
         *flagged             = 1;
     }
     void *argv[1] = {&plan.args};
-    HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, 0, (hipStream_t)hip_stream));
+    HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, plan.lds_bytes,
+                                (hipStream_t)hip_stream));
     return XCCL_OK;
 }
 
@@ -431,9 +456,10 @@ void xccl_rocm_graph_cache_destroy(void)
     }
 }
 
-void xccl_rocm_set_launch_shape(int blocks_per_cu, int cache_policy)
+void xccl_rocm_set_launch_shape(int blocks_per_cu, int cache_policy, int resident_per_cu)
 {
     read_env_once();
+    g_resident.store(resident_per_cu > 0 ? resident_per_cu : 0, std::memory_order_release);
     g_blocks_per_cu.store(blocks_per_cu > 0 ? blocks_per_cu : kDefaultBlocksPerCu, std::memory_order_release);
     g_policy.store(cache_policy == POL_PLAIN ? POL_PLAIN : POL_STREAM, std::memory_order_release);
 }
