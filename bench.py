@@ -263,6 +263,25 @@ def main():
         rot = round(nbytes / (float(np.mean(rk)) * 1e-3) / 1e9, 2)
         mc.xccl_mem_component_free(rslab, MemType.ROCM)
 
+    # Reference point: a plain 1 GiB -> 1 GiB copy kernel on the same slab (2 GiB of traffic per launch),
+    # i.e. what a 1:1 read/write stream reaches on this box.
+    copy_gbps = None
+    if nsrc >= 8 and stride * 4 >= (1 << 30):
+        gib = 1 << 30
+        for _ in range(3):
+            assert mc.bench_copy(slab + 4 * stride, slab, gib, stream) == Status.OK
+        hip.stream_synchronize(stream)
+        t0 = time.perf_counter()
+        for _ in range(20):
+            assert mc.bench_copy(slab + 4 * stride, slab, gib, stream) == Status.OK
+        hip.stream_synchronize(stream)
+        copy_gbps = round(2 * gib * 20 / (time.perf_counter() - t0) / 1e9, 2)
+        for j in range(4, 8):                   # the copy overwrote sources 4-7: restore them
+            assert mc.datagen_fill(slab + j * stride, size, Dt.FLOAT32, 2, j) == Status.OK
+        hip.device_synchronize()
+        assert mc.xccl_mem_component_reduce_multi(slab, slab + stride, dst, nsrc - 1, size, stride, Dt.FLOAT32, Op.SUM,
+                                                  MemType.ROCM) == Status.OK
+
     grid, block, name = mc._c.c_uint(0), mc._c.c_uint(0), mc._c.create_string_buffer(256)
     mc.component_lib().xccl_rocm_reduce_multi_plan(slab, slab + stride, dst, nsrc - 1, size, stride, int(Dt.FLOAT32),
                                                    int(Op.SUM), mc._c.byref(grid), mc._c.byref(block), name, 256)
@@ -281,7 +300,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(float(np.min(kms)), 4),
-                     "launches_timed": int(kms.size), "achieved_rotating_dst": rot},
+                     "launches_timed": int(kms.size), "achieved_rotating_dst": rot,
+                     "copy_kernel_GBps": copy_gbps},
     }
 
     if not a.no_cpu:

@@ -17,7 +17,8 @@
  *     src/team_lib/ucx/xccl_ucx_lib.c:631-632);
  *   - events are created once (the reference re-creates one on every record,
  *     cuda_mem_component.c:220, and leaks the old one);
- *   - small synchronous reductions go out as one hipGraph launch;
+ *   - small launches report completion through a host-mapped word the kernel
+ *     writes itself, which the host sees sooner than the queue's signal;
  *   - the vtable is extended with stream-ordered reductions whose completion
  *     is an event (see include/xccl_rocm_mem_component.h).
  *
@@ -118,8 +119,42 @@ static xccl_status_t mc_rocm_open(void)
     return XCCL_OK;
 }
 
-/* Stream, events and gate words of one device; caller holds mc_init_lock. */
-static xccl_status_t mc_rocm_device_create(mc_rocm_device_t *d)
+/* Frees whatever of a device's resources exists; caller holds mc_init_lock
+ * and has made that device current. */
+static void mc_rocm_device_destroy(mc_rocm_device_t *d)
+{
+    int i;
+
+    for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
+        if (d->events[i].hip_event != NULL) {
+            (void)hipEventDestroy(d->events[i].hip_event);
+        }
+    }
+    for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS; i++) {
+        if (d->requests[i].hip_event != NULL) {
+            (void)hipEventDestroy(d->requests[i].hip_event);
+        }
+    }
+    if (d->gate_words != NULL) {
+        (void)hipHostFree(d->gate_words);
+    }
+    if (d->flag_words != NULL) {
+        (void)hipHostFree(d->flag_words);
+    }
+    if (d->arrival_counts != NULL) {
+        (void)hipFree(d->arrival_counts);
+    }
+    if (d->gate_stream != NULL) {
+        (void)hipStreamDestroy(d->gate_stream);
+    }
+    if (d->stream != NULL) {
+        (void)hipStreamDestroy(d->stream);
+    }
+    memset(d, 0, sizeof(*d));
+}
+
+/* Stream, events and gate words of one device. */
+static xccl_status_t mc_rocm_device_create_parts(mc_rocm_device_t *d)
 {
     int i;
 
@@ -130,10 +165,11 @@ static xccl_status_t mc_rocm_device_create(mc_rocm_device_t *d)
                          hipHostMallocMapped));
     for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS; i++) {
         mc_rocm_stream_request_t *r = &d->requests[i];
-        r->flag = &d->gate_words[i];
+        r->flag  = &d->gate_words[i];
+        *r->flag = 1; /* open */
         MC_HIP(hipHostGetDevicePointer((void **)&r->dev_flag, r->flag, 0));
         MC_HIP(hipEventCreateWithFlags(&r->hip_event, hipEventDisableTiming));
-        atomic_store(&r->is_free, 1);
+        atomic_store(&r->is_free, MC_SLOT_FREE);
     }
     MC_HIP(hipHostMalloc((void **)&d->flag_words,
                          XCCL_ROCM_MC_NUM_EVENTS * MC_FLAG_STRIDE * sizeof(uint32_t),
@@ -152,9 +188,21 @@ static xccl_status_t mc_rocm_device_create(mc_rocm_device_t *d)
         ev->dev_count = d->arrival_counts + (size_t)i * (XCCL_ROCM_DONE_COUNT_BYTES / sizeof(uint32_t));
         ev->expect    = 0;
         ev->flagged   = 0;
-        atomic_store(&ev->is_free, 1);
+        atomic_store(&ev->is_free, MC_SLOT_FREE);
     }
     return XCCL_OK;
+}
+
+/* All or nothing: a device whose set-up failed half-way keeps no resources and
+ * is tried again on the next call.  Caller holds mc_init_lock. */
+static xccl_status_t mc_rocm_device_create(mc_rocm_device_t *d)
+{
+    xccl_status_t st = mc_rocm_device_create_parts(d);
+
+    if (st != XCCL_OK) {
+        mc_rocm_device_destroy(d);
+    }
+    return st;
 }
 
 /* The current device's resources, created on first use. */
@@ -437,7 +485,7 @@ static xccl_status_t mc_rocm_event_record(xccl_stream_t *stream,
     ev->stream  = hs;
     e = hipEventRecord(ev->hip_event, hs);
     if (e != hipSuccess) {
-        atomic_store(&ev->is_free, 1);
+        atomic_store(&ev->is_free, MC_SLOT_FREE);
         return XCCL_ERR_NO_MESSAGE;
     }
     ev->super.mem_type = UCS_MEMORY_TYPE_ROCM;
@@ -487,7 +535,7 @@ static xccl_status_t mc_rocm_event_free(xccl_mc_event_t *event)
     if (event == NULL) {
         return XCCL_ERR_INVALID_PARAM;
     }
-    atomic_store(&mc_rocm_event_of(event)->is_free, 1);
+    atomic_store(&mc_rocm_event_of(event)->is_free, MC_SLOT_FREE);
     return XCCL_OK;
 }
 
@@ -533,14 +581,14 @@ mc_rocm_start_stream_activity(xccl_stream_t *stream,
     __atomic_store_n(r->flag, 0, __ATOMIC_RELEASE);
     st = xccl_rocm_stream_gate(r->dev_flag, mc_gate_timeout_ns, d->gate_stream);
     if (st != XCCL_OK) {
-        atomic_store(&r->is_free, 1);
+        atomic_store(&r->is_free, MC_SLOT_FREE);
         return st;
     }
     if (hipEventRecord(r->hip_event, d->gate_stream) != hipSuccess ||
         hipStreamWaitEvent(user, r->hip_event, 0) != hipSuccess) {
         /* open the gate again: nothing may stay blocked behind a failure */
         __atomic_store_n(r->flag, 1, __ATOMIC_RELEASE);
-        atomic_store(&r->is_free, 1);
+        atomic_store(&r->is_free, MC_SLOT_FREE);
         return XCCL_ERR_NO_MESSAGE;
     }
     r->super.mem_type = UCS_MEMORY_TYPE_ROCM;
@@ -577,39 +625,37 @@ static xccl_status_t mc_rocm_get_stream(void **hip_stream)
     return XCCL_OK;
 }
 
-/* Releases the current device's resources (the reference component owns one
- * device's worth, cuda_mem_component.c:251-265). */
+/* Releases the resources of every device that was used.  (The reference
+ * component owns one device's worth, cuda_mem_component.c:251-265; this one
+ * keeps a set per device ordinal, so close visits each.) */
 static void mc_rocm_close(void)
 {
     mc_rocm_device_t *d;
-    int               dev = 0, i;
+    int               cur = 0, dev, i;
 
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MC_MAX_DEVICES) {
+    if (hipGetDevice(&cur) != hipSuccess) {
         (void)hipGetLastError();
         return;
     }
-    d = &mc_devices[dev];
     pthread_mutex_lock(&mc_init_lock);
-    if (atomic_load(&d->ready) == 1) {
+    for (dev = 0; dev < MC_MAX_DEVICES; dev++) {
+        d = &mc_devices[dev];
+        if (atomic_load(&d->ready) != 1) {
+            continue;
+        }
+        if (hipSetDevice(dev) != hipSuccess) {
+            (void)hipGetLastError();
+            continue;
+        }
         for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS; i++) {
             __atomic_store_n(d->requests[i].flag, 1, __ATOMIC_RELEASE); /* open any gate left shut */
         }
         (void)hipStreamSynchronize(d->gate_stream);
         (void)hipStreamSynchronize(d->stream);
         xccl_rocm_graph_cache_destroy();
-        for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
-            (void)hipEventDestroy(d->events[i].hip_event);
-        }
-        for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS; i++) {
-            (void)hipEventDestroy(d->requests[i].hip_event);
-        }
-        (void)hipHostFree(d->gate_words);
-        (void)hipHostFree(d->flag_words);
-        (void)hipFree(d->arrival_counts);
-        (void)hipStreamDestroy(d->gate_stream);
-        (void)hipStreamDestroy(d->stream);
-        memset(d, 0, sizeof(*d));
+        mc_rocm_device_destroy(d); /* also clears `ready` */
     }
+    (void)hipSetDevice(cur);
     pthread_mutex_unlock(&mc_init_lock);
 }
 
