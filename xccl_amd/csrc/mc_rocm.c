@@ -65,6 +65,15 @@ typedef struct mc_rocm_event {
     unsigned           polls;
 } mc_rocm_event_t;
 
+/* Spin-wait hint: keeps a polling hardware thread from starving its sibling. */
+#if defined(__x86_64__) || defined(__i386__)
+#define MC_CPU_RELAX() __builtin_ia32_pause()
+#elif defined(__aarch64__)
+#define MC_CPU_RELAX() __asm__ __volatile__("yield")
+#else
+#define MC_CPU_RELAX() ((void)0)
+#endif
+
 #define MC_FLAG_STRIDE 16 /* uint32 words between completion words: one per 64-byte line */
 
 typedef struct mc_rocm_stream_request {
@@ -319,6 +328,7 @@ static xccl_status_t mc_rocm_flag_poll(mc_rocm_event_t *ev, int block)
         if (!block) {
             return XCCL_INPROGRESS;
         }
+        MC_CPU_RELAX();
     }
 }
 
