@@ -114,6 +114,14 @@ def latency_sweep(mc, hip, iters, full):
                 row[mode] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
                              "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
             res["n%d_%dB" % (nsrc, b)] = row
+    # the memory-type probe libxccl issues at least twice per collective (mem_component.c:150-174)
+    host = np.zeros(16, dtype=np.uint8)
+    for name, ptr in (("device", buf.ptr), ("unregistered_host", host.ctypes.data)):
+        st, ns, mt = mc.bench_mem_type(ptr, 2000)
+        assert st == Status.OK
+        res["mem_type_probe_" + name] = {"p50": round(float(np.percentile(ns[200:], 50)) / 1e3, 3),
+                                         "p99": round(float(np.percentile(ns[200:], 99)) / 1e3, 3),
+                                         "answer": mt.name if mt is not None else "not recognised"}
     buf.close()
     return res
 
@@ -295,7 +303,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "reduce_multi FLOAT32 SUM, %d source vectors x %d elements at stride %d B in one slab "
                                "(radix-8 k-nomial step); stream-ordered launches" % (nsrc, size, stride),
-                   "bytes_per_step": nbytes, "device": hip.device_name(0) or "gfx950",
+                   "bytes_per_step": nbytes, "device": "gfx950 (%s)" % hip.device_name(0),
                    "kernel": name.value.decode(), "grid": grid.value, "block": block.value},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "sync_entry": {"ms_per_step": round(sync_ms, 4), "GBps": round(nbytes / sync_ms / 1e6, 2)},
@@ -322,7 +330,8 @@ def main():
         if a.latency_full:
             os.makedirs(a.out_dir, exist_ok=True)
             json.dump(lat, open(os.path.join(a.out_dir, "latency.json"), "w"), indent=1)
-            out["latency_us"] = {k: v for k, v in lat.items() if k.endswith(("_4B", "_1024B", "_32768B"))}
+            out["latency_us"] = {k: v for k, v in lat.items()
+                                 if k.endswith(("_4B", "_1024B", "_32768B")) or k.startswith("mem_type")}
         else:
             out["latency_us"] = lat
 

@@ -110,3 +110,26 @@ xccl_status_t xccl_rocm_bench_kernel_times(xccl_rocm_mem_component_t *mc, void *
     }
     return XCCL_OK;
 }
+
+/*
+ * Times `iters` mem_type probes of `ptr` (the query libxccl issues at least
+ * twice per collective, reference src/utils/mem_component.c:150-174) and
+ * stores each call's duration in ns_out; *mt_out receives the last answer
+ * (UCS_MEMORY_TYPE_LAST if the component did not recognise the pointer).
+ */
+xccl_status_t xccl_rocm_bench_mem_type(xccl_rocm_mem_component_t *mc, void *ptr, size_t iters, uint64_t *ns_out,
+                                       int *mt_out)
+{
+    ucs_memory_type_t mt = UCS_MEMORY_TYPE_LAST;
+    size_t            i;
+
+    for (i = 0; i < iters; i++) {
+        const uint64_t t0 = now_ns();
+        if (mc->super.mem_type(ptr, &mt) != XCCL_OK) {
+            mt = UCS_MEMORY_TYPE_LAST;
+        }
+        ns_out[i] = now_ns() - t0;
+    }
+    *mt_out = (int)mt;
+    return XCCL_OK;
+}

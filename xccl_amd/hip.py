@@ -142,7 +142,7 @@ def event_elapsed_ms(start: int, stop: int) -> float:
 def device_name(i: int = 0) -> str:
     buf = ctypes.create_string_buffer(256)
     check(lib().hipDeviceGetName(buf, ctypes.c_int(256), ctypes.c_int(i)), "hipDeviceGetName")
-    return buf.value.decode()
+    return buf.value.decode() or "device %d" % i     # some boxes report an empty marketing name
 
 
 def device_attribute(attr: int, dev: int = 0) -> int:

@@ -148,6 +148,7 @@ def benchkit_lib():
         lib.xccl_rocm_bench_copy.argtypes = [_vp, _vp, _sz, _vp]
         lib.xccl_rocm_bench_latency.argtypes = [_vp, _vp, _int, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
         lib.xccl_rocm_bench_kernel_times.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp]
+        lib.xccl_rocm_bench_mem_type.argtypes = [_vp, _vp, _sz, _vp, _vp]
         _datagen_lib = lib
     return _datagen_lib
 
@@ -309,6 +310,16 @@ def bench_kernel_times(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters
     for e in evs:
         hip.event_destroy(e)
     return _st(st), out
+
+
+def bench_mem_type(ptr, iters: int):
+    """Durations in ns (numpy uint64) of `iters` mem_type probes of `ptr` through the
+    component's vtable, and the memory type the last probe reported (None: not recognised)."""
+    import numpy as np
+    out = np.zeros(iters, dtype=np.uint64)
+    mt = _c.c_int(0)
+    st = benchkit_lib().xccl_rocm_bench_mem_type(_c.addressof(component()), ptr, iters, out.ctypes.data, _c.byref(mt))
+    return _st(st), out, (None if mt.value == int(MemType.LAST) else MemType(mt.value))
 
 
 # ---- UCX team-library call sites over a loopback transport (include/xccl_rocm_ucx_replay.h) ----
