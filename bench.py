@@ -122,6 +122,16 @@ def latency_sweep(mc, hip, iters, full):
         res["mem_type_probe_" + name] = {"p50": round(float(np.percentile(ns[200:], 50)) / 1e3, 3),
                                          "p99": round(float(np.percentile(ns[200:], 99)) / 1e3, 3),
                                          "answer": mt.name if mt is not None else "not recognised"}
+    # scratch per collective: mem_alloc + mem_free through the vtable, freed blocks cached (default) or not
+    for label, limit in (("cached", 8 << 30), ("runtime", 0)):
+        mc.mem_pool_set_limit(limit)
+        for nb in (64 << 10, 1 << 20, 64 << 20, 7 * 256 << 20):    # last: scratch of the headline radix-8 step
+            st, ns = mc.bench_alloc_free(nb, 300 if nb <= (64 << 20) else 60)
+            assert st == Status.OK
+            res["alloc_free_%s_%dKiB" % (label, nb >> 10)] = {
+                "p50": round(float(np.percentile(ns[10:], 50)) / 1e3, 3),
+                "p99": round(float(np.percentile(ns[10:], 99)) / 1e3, 3)}
+    mc.mem_pool_set_limit(8 << 30)
     buf.close()
     return res
 
@@ -331,7 +341,7 @@ def main():
             os.makedirs(a.out_dir, exist_ok=True)
             json.dump(lat, open(os.path.join(a.out_dir, "latency.json"), "w"), indent=1)
             out["latency_us"] = {k: v for k, v in lat.items()
-                                 if k.endswith(("_4B", "_1024B", "_32768B")) or k.startswith("mem_type")}
+                                 if k.endswith(("_4B", "_1024B", "_32768B")) or k.startswith(("mem_type", "alloc_free"))}
         else:
             out["latency_us"] = lat
 

@@ -42,6 +42,15 @@ def test_dispatcher_abi_symbols_exported():
         assert hasattr(lib, n), "libxccl_mc.so does not export %s" % n
 
 
+def test_mem_pool_abi_symbols_exported():
+    lib = mc.component_lib()
+    names = _declared_functions("xccl_rocm_mem_pool.h")
+    assert names == ["xccl_rocm_mem_pool_get_stats", "xccl_rocm_mem_pool_set_limit"]
+    for n in names:
+        assert hasattr(lib, n), "xccl_rocm_mem_component.so does not export %s" % n
+    assert ctypes.sizeof(mc.MemPoolStats) == 48
+
+
 def test_component_object_and_alias():
     """One object, two names: the reference loader dlsym()s
     "xccl_cuda_mem_component" for every memory type (mem_component.c:30)."""

@@ -52,6 +52,65 @@ def test_device_alloc_cache(rocm):
         assert rocm.xccl_mem_component_free(p, MemType.ROCM) == Status.OK
 
 
+def test_freed_scratch_is_cached_and_reused(rocm, oracle):
+    """The component's mem_free keeps blocks for the next mem_alloc of the same
+    size class (per-collective scratch, allreduce_knomial.c:181-183), a reused
+    block works as reduction scratch, and a limit of 0 restores the runtime's
+    allocate/free per call."""
+    MiB = 1 << 20
+    comp = rocm.component()
+    rocm.mem_pool_set_limit(0)                      # start from an empty cache
+    rocm.mem_pool_set_limit(64 * MiB)
+    s0 = rocm.mem_pool_stats()
+
+    def alloc(n):
+        p = ctypes.c_void_p()
+        assert comp.super.mem_alloc(ctypes.byref(p), n) == Status.OK
+        return p.value
+
+    a = alloc(3 * MiB)
+    assert rocm.xccl_mem_component_type(a) == (Status.OK, MemType.ROCM)
+    assert comp.super.mem_free(a) == Status.OK
+    s1 = rocm.mem_pool_stats()
+    assert s1.free_blocks == 1 and s1.cached_bytes == 3 * MiB and s1.misses == s0.misses + 1
+    b = alloc(3 * MiB - 100)                        # same class: the same block
+    assert b == a and rocm.mem_pool_stats().hits == s0.hits + 1
+    c = alloc(3 * MiB)                              # a second one while the first is live
+    assert c != a
+
+    # the reused block as scratch of a 4-source reduce_multi (3 vectors at stride 1 MiB)
+    n = 200_000
+    s1 = oracle.fill(n, Dt.INT32, 21, 1000)
+    s2 = np.zeros((3, MiB // 4), dtype=np.int32)
+    for j in range(3):
+        s2[j, :n] = oracle.fill(n, Dt.INT32, 21, j)
+    want = np.empty(n, dtype=np.int32)
+    oracle.reduce_multi(s1, s2, want, 3, n, MiB, Dt.INT32, Op.SUM)
+    own = hip.DeviceBuffer(n * 4)
+    dst = hip.DeviceBuffer(n * 4)
+    own.upload(s1)
+    hip.memcpy_htod(b, s2)
+    assert rocm.xccl_mem_component_reduce_multi(own.ptr, b, dst.ptr, 3, n, MiB, Dt.INT32, Op.SUM,
+                                                MemType.ROCM) == Status.OK
+    assert_same(dst.download(np.int32, n, 0), want, Dt.INT32, Op.SUM, "reduction out of a reused scratch block")
+
+    assert comp.super.mem_free(b) == Status.OK and comp.super.mem_free(c) == Status.OK
+    assert comp.super.mem_free(b) == Status.ERR_NO_MESSAGE          # freed twice: reported, nothing released
+    assert rocm.mem_pool_stats().free_blocks == 2
+    big = alloc(128 * MiB)                          # beyond the limit: never kept
+    assert comp.super.mem_free(big) == Status.OK
+    assert rocm.mem_pool_stats().free_blocks == 2
+    rocm.mem_pool_set_limit(0)
+    s2 = rocm.mem_pool_stats()
+    assert s2.free_blocks == 0 and s2.cached_bytes == 0 and s2.live_blocks == s0.live_blocks
+    d = alloc(3 * MiB)
+    assert comp.super.mem_free(d) == Status.OK
+    assert rocm.mem_pool_stats().hits == s0.hits + 1                # nothing was served from a cache
+    rocm.mem_pool_set_limit(8 << 30)
+    own.close()
+    dst.close()
+
+
 def test_event_record_query_free_and_pool(rocm):
     """Pool exhaustion is XCCL_ERR_NO_RESOURCE (cuda_mem_component.c:91,107);
     a freed slot is reusable."""

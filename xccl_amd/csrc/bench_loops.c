@@ -133,3 +133,29 @@ xccl_status_t xccl_rocm_bench_mem_type(xccl_rocm_mem_component_t *mc, void *ptr,
     *mt_out = (int)mt;
     return XCCL_OK;
 }
+
+/*
+ * Times `iters` mem_alloc(len) + mem_free pairs through the component's
+ * vtable -- what one collective pays for its scratch buffer (reference
+ * allreduce_knomial.c:181-183 and xccl_ucx_allreduce_knomial's completion) --
+ * and stores each pair's duration in ns_out.
+ */
+xccl_status_t xccl_rocm_bench_alloc_free(xccl_rocm_mem_component_t *mc, size_t len, size_t iters, uint64_t *ns_out)
+{
+    size_t i;
+
+    for (i = 0; i < iters; i++) {
+        void          *p  = NULL;
+        const uint64_t t0 = now_ns();
+        xccl_status_t  st = mc->super.mem_alloc(&p, len);
+        if (st != XCCL_OK) {
+            return st;
+        }
+        st = mc->super.mem_free(p);
+        ns_out[i] = now_ns() - t0;
+        if (st != XCCL_OK) {
+            return st;
+        }
+    }
+    return XCCL_OK;
+}

@@ -27,6 +27,8 @@
  */
 #include "xccl_rocm_kernels.h"
 #include "xccl_rocm_mem_component.h"
+#include "xccl_rocm_mem_pool.h"
+#include "mc_pool.h"
 
 #include <hip/hip_runtime_api.h>
 #include <pthread.h>
@@ -44,6 +46,10 @@
 /* Upper bound on how long a stream gate keeps a user stream blocked when
  * finish_stream_activity is never called (XCCL_MC_ROCM_GATE_TIMEOUT_MS). */
 #define MC_DEFAULT_GATE_TIMEOUT_MS 30000
+
+/* Bytes of freed device blocks mem_free may keep for the next mem_alloc
+ * (XCCL_MC_ROCM_POOL_MAX_BYTES; 0 = keep none).  Sized for a part with 288 GB. */
+#define MC_DEFAULT_POOL_MAX_BYTES ((size_t)8 << 30)
 
 /* pool slot states (`is_free` keeps the reference's member name) */
 enum { MC_SLOT_BUSY = 0, MC_SLOT_FREE = 1, MC_SLOT_DRAINING = 2 };
@@ -110,11 +116,37 @@ static uint64_t         mc_gate_timeout_ns;
         }                                                                         \
     } while (0)
 
-static xccl_status_t mc_rocm_open(void)
+static int mc_rocm_backing_alloc(void **ptr, size_t len)
+{
+    hipError_t e = hipMalloc(ptr, len);
+
+    if (e != hipSuccess) {
+        (void)hipGetLastError(); /* leave no sticky error behind */
+        return (int)e;
+    }
+    return 0;
+}
+
+static int mc_rocm_backing_free(void *ptr)
+{
+    hipError_t e = hipFree(ptr);
+
+    if (e != hipSuccess && e != hipErrorDeinitialized) {
+        (void)hipGetLastError();
+        return (int)e;
+    }
+    return 0;
+}
+
+/* Environment knobs, read once: by open() when a loader calls it, else by the
+ * first entry that needs them. */
+static pthread_once_t mc_config_once = PTHREAD_ONCE_INIT;
+
+static void mc_rocm_read_config(void)
 {
     const char *s;
+    size_t      pool_limit = MC_DEFAULT_POOL_MAX_BYTES;
 
-    /* No device call here: the process may not have chosen its GPU yet. */
     mc_graph_max_bytes = MC_DEFAULT_GRAPH_MAX_BYTES;
     s = getenv("XCCL_MC_ROCM_GRAPH_MAX_BYTES");
     if (s != NULL) {
@@ -125,6 +157,17 @@ static xccl_status_t mc_rocm_open(void)
     if (s != NULL) {
         mc_gate_timeout_ns = strtoull(s, NULL, 0) * 1000000ull;
     }
+    s = getenv("XCCL_MC_ROCM_POOL_MAX_BYTES");
+    if (s != NULL) {
+        pool_limit = (size_t)strtoull(s, NULL, 0);
+    }
+    mc_pool_configure(mc_rocm_backing_alloc, mc_rocm_backing_free, pool_limit);
+}
+
+static xccl_status_t mc_rocm_open(void)
+{
+    /* No device call here: the process may not have chosen its GPU yet. */
+    (void)pthread_once(&mc_config_once, mc_rocm_read_config);
     return XCCL_OK;
 }
 
@@ -221,6 +264,7 @@ static xccl_status_t mc_rocm_device(mc_rocm_device_t **out)
     mc_rocm_device_t *d;
     xccl_status_t     st = XCCL_OK;
 
+    (void)pthread_once(&mc_config_once, mc_rocm_read_config);
     MC_HIP(hipGetDevice(&dev));
     if (dev < 0 || dev >= MC_MAX_DEVICES) {
         return XCCL_ERR_NO_RESOURCE;
@@ -240,16 +284,53 @@ static xccl_status_t mc_rocm_device(mc_rocm_device_t **out)
     return st;
 }
 
+/* cuda_mem_component.c:34-44, with freed blocks cached (mc_pool.h). */
 static xccl_status_t mc_rocm_mem_alloc(void **ptr, size_t len)
 {
-    MC_HIP(hipMalloc(ptr, len));
+    int dev = 0, rc;
+
+    (void)pthread_once(&mc_config_once, mc_rocm_read_config);
+    MC_HIP(hipGetDevice(&dev));
+    rc = mc_pool_alloc(dev, ptr, len);
+    if (rc != 0) {
+        fprintf(stderr, "xccl mc_rocm: device allocation of %zu bytes failed with %d (%s)\n", len, rc,
+                hipGetErrorString((hipError_t)rc));
+        return XCCL_ERR_NO_MESSAGE;
+    }
     return XCCL_OK;
 }
 
 static xccl_status_t mc_rocm_mem_free(void *ptr)
 {
-    MC_HIP(hipFree(ptr));
+    int rc;
+
+    (void)pthread_once(&mc_config_once, mc_rocm_read_config);
+    rc = mc_pool_free(ptr);
+    if (rc != 0) {
+        fprintf(stderr, "xccl mc_rocm: mem_free(%p) failed with %d%s\n", ptr, rc,
+                rc < 0 ? " (block freed twice)" : "");
+        return XCCL_ERR_NO_MESSAGE;
+    }
     return XCCL_OK;
+}
+
+void xccl_rocm_mem_pool_set_limit(size_t limit_bytes)
+{
+    (void)pthread_once(&mc_config_once, mc_rocm_read_config);
+    mc_pool_set_limit(limit_bytes);
+}
+
+void xccl_rocm_mem_pool_get_stats(xccl_rocm_mem_pool_stats_t *out)
+{
+    mc_pool_stats_t st;
+
+    mc_pool_get_stats(&st);
+    out->hits          = st.hits;
+    out->misses        = st.misses;
+    out->backing_frees = st.backing_frees;
+    out->cached_bytes  = st.cached_bytes;
+    out->live_blocks   = st.live_blocks;
+    out->free_blocks   = st.free_blocks;
 }
 
 /* cuda_mem_component.c:182-204: device memory -> this component's type,
@@ -647,6 +728,7 @@ static void mc_rocm_close(void)
         (void)hipGetLastError();
         return;
     }
+    mc_pool_trim(-1);
     pthread_mutex_lock(&mc_init_lock);
     for (dev = 0; dev < MC_MAX_DEVICES; dev++) {
         d = &mc_devices[dev];

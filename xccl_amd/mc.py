@@ -149,6 +149,7 @@ def benchkit_lib():
         lib.xccl_rocm_bench_latency.argtypes = [_vp, _vp, _int, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
         lib.xccl_rocm_bench_kernel_times.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp]
         lib.xccl_rocm_bench_mem_type.argtypes = [_vp, _vp, _sz, _vp, _vp]
+        lib.xccl_rocm_bench_alloc_free.argtypes = [_vp, _sz, _sz, _vp]
         _datagen_lib = lib
     return _datagen_lib
 
@@ -320,6 +321,35 @@ def bench_mem_type(ptr, iters: int):
     mt = _c.c_int(0)
     st = benchkit_lib().xccl_rocm_bench_mem_type(_c.addressof(component()), ptr, iters, out.ctypes.data, _c.byref(mt))
     return _st(st), out, (None if mt.value == int(MemType.LAST) else MemType(mt.value))
+
+
+def bench_alloc_free(nbytes: int, iters: int):
+    """Durations in ns (numpy uint64) of `iters` mem_alloc(nbytes) + mem_free pairs
+    through the component's vtable."""
+    import numpy as np
+    out = np.zeros(iters, dtype=np.uint64)
+    st = benchkit_lib().xccl_rocm_bench_alloc_free(_c.addressof(component()), nbytes, iters, out.ctypes.data)
+    return _st(st), out
+
+
+class MemPoolStats(_c.Structure):
+    """include/xccl_rocm_mem_pool.h: xccl_rocm_mem_pool_stats_t"""
+    _fields_ = [("hits", _c.c_uint64), ("misses", _c.c_uint64), ("backing_frees", _c.c_uint64),
+                ("cached_bytes", _c.c_size_t), ("live_blocks", _c.c_size_t), ("free_blocks", _c.c_size_t)]
+
+
+def mem_pool_set_limit(limit_bytes: int) -> None:
+    fn = component_lib().xccl_rocm_mem_pool_set_limit
+    fn.argtypes, fn.restype = [_sz], None
+    fn(limit_bytes)
+
+
+def mem_pool_stats() -> MemPoolStats:
+    fn = component_lib().xccl_rocm_mem_pool_get_stats
+    fn.argtypes, fn.restype = [_c.POINTER(MemPoolStats)], None
+    out = MemPoolStats()
+    fn(_c.byref(out))
+    return out
 
 
 # ---- UCX team-library call sites over a loopback transport (include/xccl_rocm_ucx_replay.h) ----
