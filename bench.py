@@ -53,6 +53,9 @@ def parse():
     ap.add_argument("--matrix", action="store_true",
                     help="kernel GB/s of every benchmark configuration (all dtype/op pairs of the integer sweep "
                          "and the 16-source cases included); table to <out-dir>/matrix.json, nothing else")
+    ap.add_argument("--replay", action="store_true",
+                    help="time whole allreduce collectives of the replayed UCX call sites (8 loopback ranks on the one "
+                         "GPU): blocking reductions as in the reference vs stream-ordered ones, scratch cached vs not")
     ap.add_argument("--latency-full", action="store_true",
                     help="all 14 sizes x 10,000 iterations; table to <out-dir>/latency.json")
     ap.add_argument("--out-dir", default=os.path.join(ROOT, "bench_out"), help="where --matrix / --latency-full write")
@@ -182,6 +185,48 @@ def matrix(mc, hip, out_dir):
     return 0
 
 
+def replay_bench(mc, hip, out_dir):
+    """Whole-collective times of the replayed call sites.  The loopback transport moves bytes with device
+    copies, so the figures show what the reduction path and the scratch allocation contribute to a
+    collective, not what a network would."""
+    from xccl_amd.types import Dt, MemType, Op, Status
+    P = 8
+    rows = []
+    for count in (256, 16384, 1 << 20, 1 << 24):
+        nb = count * 4
+        src = [hip.DeviceBuffer(nb) for _ in range(P)]
+        dst = [hip.DeviceBuffer(nb) for _ in range(P)]
+        for r in range(P):
+            assert mc.datagen_fill(src[r].ptr, count, Dt.FLOAT32, 9, r) == Status.OK
+        hip.device_synchronize()
+        for alg, radix in (("allreduce_knomial", 4), ("allreduce_knomial", 8), ("allreduce_sra", 4)):
+            for mode, pool in (("blocking", 0), ("blocking", 8 << 30), ("stream_ordered", 8 << 30)):
+                mc.mem_pool_set_limit(pool)
+                ts = []
+                for it in range(35):
+                    t0 = time.perf_counter()
+                    st, stats = mc.replay_run(alg, [b.ptr for b in src], [b.ptr for b in dst], count, Dt.FLOAT32,
+                                              Op.SUM, radix=radix, stream_ordered=(mode == "stream_ordered"))
+                    ts.append(time.perf_counter() - t0)
+                    assert st == Status.OK, (alg, radix, mode, st)
+                ts = np.array(ts[5:]) * 1e6
+                rows.append({"alg": alg, "ranks": P, "radix": radix, "bytes_per_rank": nb, "reductions": mode,
+                             "scratch": "cached" if pool else "runtime alloc/free",
+                             "p50_us": round(float(np.percentile(ts, 50)), 1),
+                             "p90_us": round(float(np.percentile(ts, 90)), 1),
+                             "reduce_calls": stats["reduce_calls"] + stats["reduce_multi_calls"],
+                             "inflight_returns": stats["reduce_inflight_returns"]})
+                print("%-18s radix %d %9d B  %-14s %-18s p50 %9.1f us" % (alg, radix, nb, mode, rows[-1]["scratch"],
+                                                                        rows[-1]["p50_us"]), file=sys.stderr, flush=True)
+        for b in src + dst:
+            b.close()
+    mc.mem_pool_set_limit(8 << 30)
+    os.makedirs(out_dir, exist_ok=True)
+    json.dump(rows, open(os.path.join(out_dir, "replay.json"), "w"), indent=1)
+    print(json.dumps({"replay_rows": len(rows), "file": os.path.join(out_dir, "replay.json")}))
+    return 0
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -203,6 +248,8 @@ def main():
 
     if a.matrix:
         return matrix(mc, hip, a.out_dir)
+    if a.replay:
+        return replay_bench(mc, hip, a.out_dir)
 
     size, nsrc = a.size, a.nsrc
     stride = size * 4
