@@ -109,7 +109,7 @@ def latency_sweep(mc, hip, iters, full):
         for b in sizes_b:
             cnt = b // 4
             row = {}
-            for mode in ("sync", "event", "stream", "graph"):
+            for mode in ("sync", "event", "stream", "graph", "issue"):
                 st, ns = mc.bench_latency(mode, buf.ptr, buf.ptr + maxb, buf.ptr + 9 * maxb, nsrc - 1, cnt, maxb,
                                           Dt.FLOAT32, Op.SUM, iters)
                 assert st == Status.OK, (mode, st)

@@ -27,6 +27,8 @@ typedef xccl_status_t (*graph_fn_t)(void *, void *, void *, size_t, size_t, size
  *   mode 1: reduce_multi_nb on the component stream + event_query polling
  *   mode 2: `graph_fn` (xccl_rocm_reduce_multi_graph) + hipStreamSynchronize
  *   mode 3: reduce_multi_nb without event + hipStreamSynchronize
+ *   mode 4: reduce_multi_nb + event; only the call itself is timed (the host's
+ *           cost of issuing one reduction), the wait that follows is not
  * Returns the first non-OK status, or XCCL_OK.
  */
 xccl_status_t xccl_rocm_bench_latency(xccl_rocm_mem_component_t *mc, graph_fn_t graph_fn, int mode, void *sbuf1,
@@ -57,6 +59,18 @@ xccl_status_t xccl_rocm_bench_latency(xccl_rocm_mem_component_t *mc, graph_fn_t 
             if (st == XCCL_OK && hipStreamSynchronize((hipStream_t)stream) != hipSuccess) {
                 st = XCCL_ERR_NO_MESSAGE;
             }
+        } else if (mode == 4) {
+            xccl_mc_event_t *ev = NULL;
+            st        = mc->reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, NULL, &ev);
+            ns_out[i] = now_ns() - t0;
+            if (st == XCCL_OK) {
+                st = mc->event_wait(ev);
+                mc->super.event_free(ev);
+            }
+            if (st != XCCL_OK) {
+                return st;
+            }
+            continue;
         } else {
             st = mc->reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, NULL, NULL);
             if (st == XCCL_OK && hipStreamSynchronize((hipStream_t)stream) != hipSuccess) {

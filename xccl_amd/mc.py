@@ -284,7 +284,7 @@ def bench_copy(dst, src, nbytes, hip_stream=None) -> Status:
     return _st(benchkit_lib().xccl_rocm_bench_copy(dst, src, nbytes, hip_stream))
 
 
-LATENCY_MODES = {"sync": 0, "event": 1, "graph": 2, "stream": 3}
+LATENCY_MODES = {"sync": 0, "event": 1, "graph": 2, "stream": 3, "issue": 4}
 
 
 def bench_latency(mode: str, sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters: int):
