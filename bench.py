@@ -175,8 +175,16 @@ def matrix(mc, hip, out_dir):
         rows.append({"config": name, "dtype": dt.name, "op": op.name, "nsrc": nsrc, "size": size, "bytes": nb,
                      "kernel_ms": round(ms, 4), "GBps": round(nb / ms / 1e6, 1),
                      "frac_of_peak": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 3)})
-        print("%-8s %-8s %-5s N=%-2d size=%-9d %8.4f ms %8.1f GB/s" % (name, dt.name, op.name, nsrc, size, ms,
-                                                                      rows[-1]["GBps"]), file=sys.stderr, flush=True)
+        if name == "sweep":     # what a caller of the blocking entry sees per call, host clock
+            st, ns = mc.bench_latency("sync", buf, buf + stride, buf + nsrc * stride, nsrc - 1, size, stride, dt, op,
+                                      200)
+            assert st == Status.OK
+            rows[-1]["blocking_call_us"] = round(float(np.percentile(ns[20:], 50)) / 1e3, 2)
+            rows[-1]["blocking_call_GBps"] = round(nb / rows[-1]["blocking_call_us"] / 1e3, 1)
+        print("%-8s %-8s %-5s N=%-2d size=%-9d %8.4f ms %8.1f GB/s %s" % (
+            name, dt.name, op.name, nsrc, size, ms, rows[-1]["GBps"],
+            "blocking call %.2f us" % rows[-1]["blocking_call_us"] if name == "sweep" else ""),
+            file=sys.stderr, flush=True)
     mc.xccl_mem_component_free(buf, MemType.ROCM)
     os.makedirs(out_dir, exist_ok=True)
     json.dump(rows, open(os.path.join(out_dir, "matrix.json"), "w"), indent=1)

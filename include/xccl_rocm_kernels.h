@@ -57,16 +57,19 @@ xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf,
                                           xccl_op_t op, void *hip_stream);
 
 /*
- * xccl_rocm_reduce_multi_impl with a completion word: when the launch is small
- * (a few hundred workgroups at most) the kernel itself stores `seq` to
- * `*dev_flag` -- the device view of a host-mapped 32-bit word -- after its
+ * xccl_rocm_reduce_multi_impl with a completion word: `seq` is stored to
+ * `*dev_flag` -- the device view of a host-mapped 32-bit word -- once the
  * last result store is visible system-wide, and `*flagged` is set to 1; the
- * caller may then poll the host view of the word instead of the stream.
- * `dev_count` points at XCCL_ROCM_DONE_COUNT_BYTES of zeroed device memory the
- * workgroups count arrivals in (two levels, one counter per 128-byte line);
- * the kernel leaves it zero again.  One launch at a time per (count, flag)
- * pair.  For larger launches nothing is attached, `*flagged` is 0 and the
- * caller waits for the stream as usual.  No counterpart in the reference.
+ * caller may then poll the host view of the word instead of the stream (the
+ * host sees the word 3-5 us before the queue's completion signal).  A launch
+ * of up to 8192 workgroups writes the word itself: its workgroups count their
+ * arrivals in `dev_count`, XCCL_ROCM_DONE_COUNT_BYTES of zeroed device memory
+ * (two levels, one counter per 128-byte line), which the kernel leaves zero
+ * again.  Behind a larger launch a one-lane kernel is queued that stores the
+ * word (XCCL_MC_ROCM_TAIL_FLAG=0 in the environment turns that off; then, or
+ * if that second launch fails, `*flagged` is 0 and the caller waits for the
+ * stream as usual).  One launch at a time per (count, flag) pair.  No
+ * counterpart in the reference.
  */
 #define XCCL_ROCM_DONE_COUNT_BYTES ((1 + 64) * 128)
 xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbuf,

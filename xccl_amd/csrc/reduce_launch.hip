@@ -27,6 +27,7 @@ constexpr size_t kLdsPerCu      = 160 * 1024;
 std::atomic<int> g_blocks_per_cu{-1}; // -1: not read from the environment yet
 std::atomic<int> g_policy{-1};
 std::atomic<int> g_resident{0};
+std::atomic<int> g_tail_flag{1};
 std::atomic<int> g_cu_count[kMaxDevices];
 
 void read_env_once()
@@ -37,6 +38,8 @@ void read_env_once()
     const char *pol = getenv("XCCL_MC_ROCM_CACHE_POLICY");
     const char *bpc = getenv("XCCL_MC_ROCM_BLOCKS_PER_CU");
     const char *res = getenv("XCCL_MC_ROCM_RESIDENT_PER_CU");
+    const char *tf  = getenv("XCCL_MC_ROCM_TAIL_FLAG");
+    g_tail_flag.store(tf ? atoi(tf) != 0 : 1, std::memory_order_release);
     int         v   = bpc ? atoi(bpc) : 0;
     g_resident.store(res && atoi(res) > 0 ? atoi(res) : 0, std::memory_order_release);
     g_policy.store((pol && atoi(pol) == POL_PLAIN) ? POL_PLAIN : POL_STREAM, std::memory_order_release);
@@ -354,6 +357,14 @@ xccl_status_t graph_launch(Plan &plan, hipStream_t stream)
     return XCCL_OK;
 }
 
+// Completion word of a launch too large to count its own workgroups: a
+// one-lane kernel queued right behind it.  Stream order makes it start after
+// the reduction has finished and its results are visible system-wide.
+__global__ void tail_flag_kernel(uint32_t *flag, uint32_t seq)
+{
+    __hip_atomic_store(flag, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // Polls *flag (host-mapped) from one lane; see xccl_rocm_stream_gate.
 __global__ void stream_gate_kernel(int *flag, uint64_t max_ticks)
 {
@@ -404,15 +415,24 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
     if (st != XCCL_OK) {
         return st;
     }
-    if (dev_count != nullptr && dev_flag != nullptr && flagged != nullptr && plan.grid <= kMaxFlaggedGrid) {
+    const bool want_flag = dev_count != nullptr && dev_flag != nullptr && flagged != nullptr;
+    const bool in_kernel = want_flag && plan.grid <= kMaxFlaggedGrid;
+    if (in_kernel) {
         plan.args.done_seq   = seq;
         plan.args.done_count = dev_count;
         plan.args.done_flag  = dev_flag;
-        *flagged             = 1;
     }
     void *argv[1] = {&plan.args};
     HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, plan.lds_bytes,
                                 (hipStream_t)hip_stream));
+    if (in_kernel) {
+        *flagged = 1;
+    } else if (want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0) {
+        hipLaunchKernelGGL(tail_flag_kernel, dim3(1), dim3(1), 0, (hipStream_t)hip_stream, dev_flag, seq);
+        if (hipGetLastError() == hipSuccess) {
+            *flagged = 1; // otherwise the caller waits for the stream, which still works
+        }
+    }
     return XCCL_OK;
 }
 
