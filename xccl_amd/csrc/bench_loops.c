@@ -173,3 +173,37 @@ xccl_status_t xccl_rocm_bench_alloc_free(xccl_rocm_mem_component_t *mc, size_t l
     }
     return XCCL_OK;
 }
+
+/*
+ * One pair of timing events around `iters` stream-ordered reduce_multi calls
+ * enqueued back to back on the component stream: *ms_out is the whole
+ * region's device time, so region / iters is the average launch duration
+ * without a per-launch event's own cost (about 5 us per pair on this part).
+ */
+xccl_status_t xccl_rocm_bench_region_time(xccl_rocm_mem_component_t *mc, void *sbuf1, void *sbuf2, void *rbuf,
+                                          size_t count, size_t size, size_t stride, xccl_dt_t dtype, xccl_op_t op,
+                                          size_t iters, void *ev_begin, void *ev_end, float *ms_out)
+{
+    void         *stream = NULL;
+    xccl_status_t st     = mc->get_stream(&stream);
+    size_t        i;
+
+    if (st != XCCL_OK) {
+        return st;
+    }
+    if (hipEventRecord((hipEvent_t)ev_begin, (hipStream_t)stream) != hipSuccess) {
+        return XCCL_ERR_NO_MESSAGE;
+    }
+    for (i = 0; i < iters; i++) {
+        st = mc->reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, NULL, NULL);
+        if (st != XCCL_OK) {
+            return st;
+        }
+    }
+    if (hipEventRecord((hipEvent_t)ev_end, (hipStream_t)stream) != hipSuccess ||
+        hipStreamSynchronize((hipStream_t)stream) != hipSuccess ||
+        hipEventElapsedTime(ms_out, (hipEvent_t)ev_begin, (hipEvent_t)ev_end) != hipSuccess) {
+        return XCCL_ERR_NO_MESSAGE;
+    }
+    return XCCL_OK;
+}

@@ -148,6 +148,7 @@ def benchkit_lib():
         lib.xccl_rocm_bench_copy.argtypes = [_vp, _vp, _sz, _vp]
         lib.xccl_rocm_bench_latency.argtypes = [_vp, _vp, _int, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
         lib.xccl_rocm_bench_kernel_times.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp]
+        lib.xccl_rocm_bench_region_time.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp, _vp]
         lib.xccl_rocm_bench_mem_type.argtypes = [_vp, _vp, _sz, _vp, _vp]
         lib.xccl_rocm_bench_alloc_free.argtypes = [_vp, _sz, _sz, _vp]
         _datagen_lib = lib
@@ -311,6 +312,19 @@ def bench_kernel_times(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters
     for e in evs:
         hip.event_destroy(e)
     return _st(st), out
+
+
+def bench_region_time(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters: int):
+    """Device time in ms of `iters` back-to-back launches on the component stream,
+    from ONE pair of HIP events around them all."""
+    from . import hip
+    e0, e1 = hip.event_create(), hip.event_create()
+    ms = _c.c_float(0)
+    st = benchkit_lib().xccl_rocm_bench_region_time(_c.addressof(component()), sbuf1, sbuf2, rbuf, count, size, stride,
+                                                    int(dtype), int(op), iters, e0, e1, _c.byref(ms))
+    hip.event_destroy(e0)
+    hip.event_destroy(e1)
+    return _st(st), ms.value
 
 
 def bench_mem_type(ptr, iters: int):
