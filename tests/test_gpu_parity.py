@@ -187,10 +187,11 @@ def test_unsupported_returns_status_and_writes_nothing(rocm):
     buf.close()
 
 
-@pytest.mark.parametrize("n2", [1, 2, 3, 4, 5, 6, 7, 8, 9, 14, 15, 16, 17, 31, 32])
+@pytest.mark.parametrize("n2", [1, 2, 3, 4, 5, 6, 7, 8, 9, 14, 15, 16, 17, 31, 32, 100, 1000])
 def test_source_counts(rocm, oracle, n2):
     """MAX_REQS = 32 caps the k-nomial radix at 17 (xccl_ucx_lib.h:65); cover
-    every count up to there and a little beyond, fp32 SUM and fp64 MAX."""
+    every count up to there and far beyond (the any-count kernel), fp32 SUM,
+    fp64 MAX and int16 PROD."""
     run_and_check(rocm, oracle, Dt.FLOAT32, Op.SUM, 6007, n2, seed=20 + n2)
     run_and_check(rocm, oracle, Dt.FLOAT64, Op.MAX, 1501, n2, seed=40 + n2)
     run_and_check(rocm, oracle, Dt.INT16, Op.PROD, 2503, n2, seed=60 + n2)
