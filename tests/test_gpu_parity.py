@@ -24,7 +24,7 @@ def _id(p):
 def test_every_dtype_op_small(rocm, oracle, pair):
     """Every supported (dtype, op): source counts on and off the specialised
     kernels (2, 3, 4, 8, 16 sources vs 5, 9, 17), sizes around the 16-byte
-    vector and the 256-lane tile."""
+    vector and the 128-vector tile of a one-wave workgroup."""
     dt, op = pair
     for n2, size in ((1, 1), (1, 1000), (2, 37), (3, 4099), (4, 513), (7, 2048 + 5), (8, 700), (15, 1031),
                      (16, 129)):
@@ -198,8 +198,9 @@ def test_source_counts(rocm, oracle, n2):
 
 
 def test_grid_cap_and_ragged_tiles(rocm, oracle):
-    """Sizes that leave a partial tile, with the persistent grid capped low so
-    every block loops, and uncapped so every block runs once."""
+    """Sizes that leave a partial tile, with the grid capped low (1 and 64
+    workgroups per compute unit) so that every workgroup loops over tiles, then
+    the other cache policy without a residency cap."""
     lib = rocm.component_lib()
     try:
         for bpc in (1, 64):
