@@ -294,3 +294,23 @@ def test_init_rejects_null_and_missing_dir():
 def test_libs_are_in_tree():
     for n in ("xccl_rocm_mem_component.so", "libxccl_mc.so", "libxccl_rocm_benchkit.so"):
         assert os.path.isfile(os.path.join(LIB_DIR, n))
+
+
+def test_cached_buffer_is_never_lent_twice(fake, tmp_path):
+    """Collectives may be posted from several threads (the ucx team library
+    advertises XCCL_THREAD_MODE_MULTIPLE, xccl_ucx_lib.c:631-632): 8 threads
+    borrow and return small buffers through the dispatcher; nobody may ever
+    find another thread's bytes in the buffer it holds."""
+    out = str(tmp_path / "libdispatch_stress.so")
+    subprocess.run(["gcc", "-shared", "-fPIC", "-O2", "-Wall", "-Wextra", "-Werror", "-I", INC, "-o", out,
+                    os.path.join(ROOT, "tests", "dispatch_stress.c"), "-L", LIB_DIR, "-lxccl_mc", "-lpthread",
+                    "-Wl,-rpath," + LIB_DIR], check=True)
+    mc.dispatch_lib()                                   # the copy of libxccl_mc.so the fixture initialised
+    lib = ctypes.CDLL(out)
+    lib.dispatch_stress.restype = ctypes.c_long
+    loans = ctypes.c_long(0)
+    errors = lib.dispatch_stress(8, 200000, int(MemType.CUDA), ctypes.byref(loans))
+    assert errors == 0
+    assert loans.value > 0                              # the cached buffer did go round
+    vt = mc.dispatch_lib().xccl_mem_component_get(int(MemType.CUDA)).contents
+    assert vt.cache.used == 0

@@ -12,6 +12,9 @@
  *     (mem_component.c:30 dereferences a NULL dlsym result);
  *   - stream_to_mem_type knows XCCL_STREAM_TYPE_ROCM (mem_component.c:176-178
  *     has the CUDA entry only);
+ *   - the cached buffer is claimed atomically (mem_component.c:68-82 tests and
+ *     sets `used` without synchronisation although collectives may be posted
+ *     from several threads);
  *   - the *_nb / event_wait entries forward to the component's extension.
  */
 #include "xccl_rocm_mem_component.h"
@@ -135,17 +138,25 @@ xccl_status_t xccl_mem_component_alloc(void **ptr, size_t len, ucs_memory_type_t
     }
     /* One buffer of cache.size bytes stays allocated and is lent to whichever
      * request fits and finds it idle: the k-nomial scratch of small messages
-     * then costs no device allocation (allreduce_knomial.c:181-183). */
-    if (mc->cache.used == 0 && mc->cache.size >= len) {
-        if (mc->cache.buf == NULL) {
-            st = mc->mem_alloc(&mc->cache.buf, mc->cache.size);
-            if (st != XCCL_OK) {
-                return st;
+     * then costs no device allocation (allreduce_knomial.c:181-183).  `used`
+     * is claimed atomically: collectives may be posted from several threads
+     * (XCCL_THREAD_MODE_MULTIPLE), and two of them must never be lent the
+     * same buffer. */
+    if (mc->cache.size >= len) {
+        int idle = 0;
+        if (__atomic_compare_exchange_n(&mc->cache.used, &idle, 1, 0, __ATOMIC_ACQ_REL, __ATOMIC_ACQUIRE)) {
+            void *buf = __atomic_load_n(&mc->cache.buf, __ATOMIC_ACQUIRE);
+            if (buf == NULL) {
+                st = mc->mem_alloc(&buf, mc->cache.size);
+                if (st != XCCL_OK) {
+                    __atomic_store_n(&mc->cache.used, 0, __ATOMIC_RELEASE);
+                    return st;
+                }
+                __atomic_store_n(&mc->cache.buf, buf, __ATOMIC_RELEASE);
             }
+            *ptr = buf;
+            return XCCL_OK;
         }
-        *ptr           = mc->cache.buf;
-        mc->cache.used = 1;
-        return XCCL_OK;
     }
     return mc->mem_alloc(ptr, len);
 }
@@ -163,8 +174,8 @@ xccl_status_t xccl_mem_component_free(void *ptr, ucs_memory_type_t mt)
     if (mc == NULL) {
         return XCCL_ERR_UNSUPPORTED;
     }
-    if (ptr == mc->cache.buf) {
-        mc->cache.used = 0;
+    if (ptr != NULL && ptr == __atomic_load_n(&mc->cache.buf, __ATOMIC_ACQUIRE)) {
+        __atomic_store_n(&mc->cache.used, 0, __ATOMIC_RELEASE);
         return XCCL_OK;
     }
     return mc->mem_free(ptr);
@@ -349,7 +360,7 @@ void xccl_mem_component_free_cache(void)
         if (mc == NULL) {
             continue;
         }
-        if (mc->cache.buf != NULL && !mc->cache.used) {
+        if (mc->cache.buf != NULL && !__atomic_load_n(&mc->cache.used, __ATOMIC_ACQUIRE)) {
             mc->mem_free(mc->cache.buf);
             mc->cache.buf = NULL;
         }
