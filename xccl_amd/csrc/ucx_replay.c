@@ -344,10 +344,17 @@ typedef struct rank_state {
 
 static xccl_status_t post(ctx_t *c, rank_state_t *s, int is_send, int peer, void *buf, size_t len)
 {
+    lb_req_t     *req = NULL;
+    xccl_status_t st;
+
     if (s->nreqs >= MAX_REQS) {
         return XCCL_ERR_NO_RESOURCE;
     }
-    return tr_post(&c->tr, is_send, s->rank, peer, buf, len, &s->reqs[s->nreqs++]);
+    st = tr_post(&c->tr, is_send, s->rank, peer, buf, len, &req);
+    if (req != NULL) {
+        s->reqs[s->nreqs++] = req; /* tracked even if its copy failed, so that the slot is released */
+    }
+    return st;
 }
 
 /* XCCL_OK when every posted request of the rank has completed (they are
