@@ -139,6 +139,24 @@ def test_enum_values_match_reference_headers():
     assert [n for n, _ in mc.MemComponentVtable._fields_] == ref_members
 
 
+def test_plan_rejects_bad_arguments_without_a_device():
+    """Argument checks come before any device query: NULL operands, a vector
+    count beyond 32 bits and an element count whose byte size would wrap are
+    XCCL_ERR_INVALID_PARAM, an unsupported pair XCCL_ERR_UNSUPPORTED."""
+    lib = mc.component_lib()
+    plan = lib.xccl_rocm_reduce_multi_plan
+    plan.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_size_t] * 3 + [ctypes.c_int] * 2 + [ctypes.c_void_p] * 3 + \
+                    [ctypes.c_size_t]
+    ok = (0x1000, 0x2000, 0x3000)
+    assert plan(None, ok[1], ok[2], 1, 16, 64, int(Dt.INT32), int(Op.SUM), None, None, None, 0) == Status.ERR_INVALID_PARAM
+    assert plan(ok[0], None, ok[2], 1, 16, 64, int(Dt.INT32), int(Op.SUM), None, None, None, 0) == Status.ERR_INVALID_PARAM
+    assert plan(ok[0], ok[1], None, 1, 16, 64, int(Dt.INT32), int(Op.SUM), None, None, None, 0) == Status.ERR_INVALID_PARAM
+    assert plan(*ok, 1 << 32, 16, 64, int(Dt.INT32), int(Op.SUM), None, None, None, 0) == Status.ERR_INVALID_PARAM
+    assert plan(*ok, 1, (1 << 56) + 1, 64, int(Dt.INT32), int(Op.SUM), None, None, None, 0) == Status.ERR_INVALID_PARAM
+    assert plan(*ok, 1, 16, 64, int(Dt.FLOAT32), int(Op.BAND), None, None, None, 0) == Status.ERR_UNSUPPORTED
+    assert plan(*ok, 1, 16, 64, int(Dt.INT128), int(Op.SUM), None, None, None, 0) == Status.ERR_UNSUPPORTED
+
+
 def test_dt_size():
     assert [dt_size(d) for d in (Dt.INT8, Dt.INT16, Dt.INT32, Dt.INT64, Dt.INT128, Dt.UINT8, Dt.UINT16, Dt.UINT32,
                                  Dt.UINT64, Dt.UINT128, Dt.FLOAT16, Dt.FLOAT32, Dt.FLOAT64, Dt.LAST_PREDEFINED,

@@ -183,8 +183,8 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     if (s1 == nullptr || s2 == nullptr || dst == nullptr) {
         return XCCL_ERR_INVALID_PARAM;
     }
-    if (count > 0xffffffffu) {
-        return XCCL_ERR_INVALID_PARAM;
+    if (count > 0xffffffffu || size > ((size_t)1 << 56)) {
+        return XCCL_ERR_INVALID_PARAM; // byte counts and vector indices below stay far from wrapping
     }
     read_env_once();
     int cus = 0;
