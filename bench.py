@@ -79,18 +79,29 @@ def cpu_baseline(size, nsrc):
 
     run(1)
     t1 = []
-    while sum(t1) < 8.0 and len(t1) < 10:
+    while sum(t1) < 8.0 and len(t1) < 60:
         t1.append(run(1))
     run(threads)
     tm = []
     while sum(tm) < 4.0 and len(tm) < 10:
         tm.append(run(threads))
     med1, medm = float(np.median(t1)), float(np.median(tm))
+    # the reference's own CPU-runnable case: xccl_dt_reduce on two 4 MiB fp32 vectors, one thread
+    n1 = 1 << 20
+    a1, b1, o1 = o.fill(n1, Dt.FLOAT32, 0, 0), o.fill(n1, Dt.FLOAT32, 0, 1), np.empty(n1, dtype=np.float32)
+    tc = []
+    for _ in range(200):
+        t0 = time.perf_counter()
+        o.dt_reduce(a1, b1, o1, n1, Dt.FLOAT32, Op.SUM)
+        tc.append(time.perf_counter() - t0)
+    medc = float(np.median(tc[20:]))
     return {
         "value": round(nbytes / med1 / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
         "sample": "%d calls of the full workload (%d x %d fp32, %d B/call), median %.1f ms/call; host traffic is "
                   "3*(N-1)*size*4 B/call" % (len(t1), nsrc, size, nbytes, med1 * 1e3),
         "all_cores": {"value": round(nbytes / medm / 1e9, 3), "cores": threads, "ms_per_call": round(medm * 1e3, 2)},
+        "two_source_1Mi_fp32": {"value": round(3 * n1 * 4 / medc / 1e9, 3), "cores": 1,
+                                "us_per_call": round(medc * 1e6, 1)},
     }, slab, out
 
 
