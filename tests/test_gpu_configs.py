@@ -56,6 +56,16 @@ def test_config3_integer_sweep(rocm, oracle, dt):
     _full_case(rocm, oracle, dt, list(INT_OPS), 4, 16777216, seed=3)
 
 
+@pytest.mark.parametrize("dt", [Dt.UINT8, Dt.UINT16, Dt.FLOAT16, Dt.FLOAT32, Dt.FLOAT64], ids=lambda d: Dt(d).name)
+def test_remaining_dtypes_every_operator_multi_megabyte(rocm, oracle, dt):
+    """The element types the integer sweep leaves out, every operator each
+    supports, 3 sources x (4 Mi + 37) elements: thousands of workgroups, a
+    ragged last tile, and launches on either side of the completion-word
+    switch depending on the element size."""
+    ops = list(INT_OPS) if int(dt) < int(Dt.FLOAT16) else [Op.MAX, Op.MIN, Op.SUM, Op.PROD]
+    _full_case(rocm, oracle, dt, ops, 3, (4 << 20) + 37, seed=6)
+
+
 @pytest.mark.parametrize("dt", [Dt.FLOAT16, Dt.FLOAT64], ids=lambda d: Dt(d).name)
 def test_config4_fp16_fp64_16_sources(rocm, oracle, dt):
     """16 sources (radix-16 step) x 33,554,432 elements, SUM/MAX/MIN.  MAX/MIN
