@@ -162,6 +162,7 @@ def matrix(mc, hip, out_dir):
     cases += [("extra", Dt.FLOAT32, Op.SUM, n, 67108864) for n in (2, 3, 4, 5, 16)]
     cases += [("extra", Dt.UINT8, op, 4, 67108864) for op in (Op.SUM, Op.MAX)]
     cases += [("extra", Dt.FLOAT16, Op.PROD, 8, 67108864), ("extra", Dt.FLOAT32, Op.MAX, 8, 67108864)]
+    cases += [("inplace", Dt.FLOAT32, Op.MAX, n, 67108864) for n in (4, 8)]
     # message-size sweep: where the call leaves the launch-bound regime and reaches the bandwidth plateau
     cases += [("sweep", Dt.FLOAT32, Op.SUM, n, 1 << k) for n in (2, 4, 8) for k in range(14, 27, 2)]
     rows = []
@@ -179,7 +180,9 @@ def matrix(mc, hip, out_dir):
                 assert mc.datagen_fill(buf + j * stride, size, dt, 3, j, key[3]) == Status.OK
             hip.device_synchronize()
             cur = key
-        st, k = mc.bench_kernel_times(buf, buf + stride, buf + nsrc * stride, nsrc - 1, size, stride, dt, op, 12)
+        # "inplace": rbuf == sbuf1, the form every k-nomial round after the first has (allreduce_knomial.c:118-121)
+        rbuf = buf if name == "inplace" else buf + nsrc * stride
+        st, k = mc.bench_kernel_times(buf, buf + stride, rbuf, nsrc - 1, size, stride, dt, op, 12)
         assert st == Status.OK
         ms = float(np.mean(k[2:]))
         nb = (nsrc + 1) * size * es
@@ -199,7 +202,7 @@ def matrix(mc, hip, out_dir):
     mc.xccl_mem_component_free(buf, MemType.ROCM)
     os.makedirs(out_dir, exist_ok=True)
     json.dump(rows, open(os.path.join(out_dir, "matrix.json"), "w"), indent=1)
-    print(json.dumps({"matrix_rows": len(rows), "min_GBps": min(r["GBps"] for r in rows if r["config"] not in ("config1", "sweep")),
+    print(json.dumps({"matrix_rows": len(rows), "min_GBps": min(r["GBps"] for r in rows if r["config"] not in ("config1", "sweep", "inplace")),
                       "file": os.path.join(out_dir, "matrix.json")}))
     return 0
 
