@@ -66,9 +66,11 @@ xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf,
  * arrivals in `dev_count`, XCCL_ROCM_DONE_COUNT_BYTES of zeroed device memory
  * (two levels, one counter per 128-byte line), which the kernel leaves zero
  * again.  Behind a larger launch a one-lane kernel is queued that stores the
- * word (XCCL_MC_ROCM_TAIL_FLAG=0 in the environment turns that off; then, or
- * if that second launch fails, `*flagged` is 0 and the caller waits for the
- * stream as usual).  One launch at a time per (count, flag) pair.  No
+ * word, provided every result store of that launch is a write-through vector
+ * store (no peeled head or tail elements: 16-byte-aligned operands and a
+ * byte count that is a multiple of 16; streaming cache policy).  Otherwise, or
+ * with XCCL_MC_ROCM_TAIL_FLAG=0 in the environment, or if that second launch
+ * fails, `*flagged` is 0 and the caller waits for the stream as usual.  One launch at a time per (count, flag) pair.  No
  * counterpart in the reference.
  */
 #define XCCL_ROCM_DONE_COUNT_BYTES ((1 + 64) * 128)

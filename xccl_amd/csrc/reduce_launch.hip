@@ -427,7 +427,12 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
                                 (hipStream_t)hip_stream));
     if (in_kernel) {
         *flagged = 1;
-    } else if (want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0) {
+    } else if (want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0 && plan.args.head + plan.args.tail == 0 &&
+               g_policy.load(std::memory_order_relaxed) == POL_STREAM) {
+        // Only when every result store of the launch is a write-through vector store: those are in
+        // memory when the reduction kernel ends.  Peeled head/tail elements (and everything under the
+        // default cache policy) may still sit dirty in an L2 until the runtime's own release at a
+        // stream synchronisation, so such launches keep completing through the stream.
         hipLaunchKernelGGL(tail_flag_kernel, dim3(1), dim3(1), 0, (hipStream_t)hip_stream, dev_flag, seq);
         if (hipGetLastError() == hipSuccess) {
             *flagged = 1; // otherwise the caller waits for the stream, which still works
