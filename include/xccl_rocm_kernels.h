@@ -61,15 +61,17 @@ xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf,
  * `*dev_flag` -- the device view of a host-mapped 32-bit word -- once the
  * last result store is visible system-wide, and `*flagged` is set to 1; the
  * caller may then poll the host view of the word instead of the stream (the
- * host sees the word 3-5 us before the queue's completion signal).  A launch
- * of up to 8192 workgroups writes the word itself: its workgroups count their
- * arrivals in `dev_count`, XCCL_ROCM_DONE_COUNT_BYTES of zeroed device memory
- * (two levels, one counter per 128-byte line), which the kernel leaves zero
- * again.  Behind a larger launch a one-lane kernel is queued that stores the
- * word, provided every result store of that launch is a write-through vector
- * store (no peeled head or tail elements: 16-byte-aligned operands and a
- * byte count that is a multiple of 16; streaming cache policy).  Otherwise, or
- * with XCCL_MC_ROCM_TAIL_FLAG=0 in the environment, or if that second launch
+ * host sees the word 3-5 us before the queue's completion signal).  A small
+ * launch writes the word itself: its workgroups count their arrivals in
+ * `dev_count`, XCCL_ROCM_DONE_COUNT_BYTES of zeroed device memory (two
+ * levels, one counter per 128-byte line), which the kernel leaves zero again.
+ * Behind a larger launch (more than 1024 workgroups; XCCL_MC_ROCM_MAX_COUNTED_GRID)
+ * a one-lane kernel is queued that stores the word, provided every result
+ * store of that launch is a write-through vector store (no peeled head or
+ * tail elements: 16-byte-aligned operands and a byte count that is a multiple
+ * of 16; streaming cache policy); launches that are not keep counting up to
+ * 8192 workgroups.  Beyond that, or with XCCL_MC_ROCM_TAIL_FLAG=0 in the
+ * environment where the queued kernel would be used, or if its launch
  * fails, `*flagged` is 0 and the caller waits for the stream as usual.  One launch at a time per (count, flag) pair.  No
  * counterpart in the reference.
  */

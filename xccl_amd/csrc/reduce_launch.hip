@@ -24,10 +24,18 @@ constexpr int kDefaultBlocksPerCu = 8192;
 constexpr int    kNoResidentCap = 32;
 constexpr size_t kLdsPerCu      = 160 * 1024;
 
+// Launches of at most this many workgroups may count their own arrivals for a
+// completion word: each workgroup pays an atomic on one of 64 shared counters
+// (~12 ns per arrival on the same word, measured), which beats the queue's
+// completion signal up to here and would serialise a grid of hundreds of
+// thousands.
+constexpr unsigned kMaxFlaggedGrid = 8192;
+
 std::atomic<int> g_blocks_per_cu{-1}; // -1: not read from the environment yet
 std::atomic<int> g_policy{-1};
 std::atomic<int> g_resident{0};
 std::atomic<int> g_tail_flag{1};
+std::atomic<unsigned> g_max_counted_grid{1024}; // measured: counting wins up to ~512 workgroups, ties at 2048, loses 3-5 % at 8192
 std::atomic<int> g_cu_count[kMaxDevices];
 
 void read_env_once()
@@ -40,6 +48,10 @@ void read_env_once()
     const char *res = getenv("XCCL_MC_ROCM_RESIDENT_PER_CU");
     const char *tf  = getenv("XCCL_MC_ROCM_TAIL_FLAG");
     g_tail_flag.store(tf ? atoi(tf) != 0 : 1, std::memory_order_release);
+    const char *mcg = getenv("XCCL_MC_ROCM_MAX_COUNTED_GRID");
+    if (mcg != nullptr && atoi(mcg) >= 0 && (unsigned)atoi(mcg) <= kMaxFlaggedGrid) {
+        g_max_counted_grid.store((unsigned)atoi(mcg), std::memory_order_release);
+    }
     int         v   = bpc ? atoi(bpc) : 0;
     g_resident.store(res && atoi(res) > 0 ? atoi(res) : 0, std::memory_order_release);
     g_policy.store((pol && atoi(pol) == POL_PLAIN) ? POL_PLAIN : POL_STREAM, std::memory_order_release);
@@ -230,11 +242,6 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     return XCCL_OK;
 }
 
-// Launches of at most this many workgroups may carry a completion word: each
-// workgroup pays an atomic on one of 64 shared counters (~12 ns per arrival
-// on the same word, measured), which beats the queue's completion signal up
-// to here and would serialise a grid of hundreds of thousands.
-constexpr unsigned kMaxFlaggedGrid = 8192;
 static_assert(XCCL_ROCM_DONE_COUNT_BYTES == (1 + kDoneShards) * kDoneStride * sizeof(uint32_t), "counter block size");
 
 // ---- single-kernel-node graph cache ---------------------------------------
@@ -415,8 +422,19 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
     if (st != XCCL_OK) {
         return st;
     }
-    const bool want_flag = dev_count != nullptr && dev_flag != nullptr && flagged != nullptr;
-    const bool in_kernel = want_flag && plan.grid <= kMaxFlaggedGrid;
+    // Who writes the completion word: the launch itself, counting its workgroups (cheapest for small
+    // grids), or a one-lane kernel queued behind it (cheaper from about a thousand workgroups on).  The
+    // second needs every result store of the launch to be a write-through vector store: those are in
+    // memory when the reduction kernel ends, while peeled head/tail elements (and everything under the
+    // default cache policy) may sit dirty in an L2 until the runtime's own release at a stream
+    // synchronisation -- such launches count up to the larger bound and beyond it complete through the
+    // stream.
+    const bool     want_flag = dev_count != nullptr && dev_flag != nullptr && flagged != nullptr;
+    const bool     tail_ok   = want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0 &&
+                               plan.args.head + plan.args.tail == 0 &&
+                               g_policy.load(std::memory_order_relaxed) == POL_STREAM;
+    const unsigned counted   = tail_ok ? g_max_counted_grid.load(std::memory_order_relaxed) : kMaxFlaggedGrid;
+    const bool     in_kernel = want_flag && plan.grid <= counted;
     if (in_kernel) {
         plan.args.done_seq   = seq;
         plan.args.done_count = dev_count;
@@ -427,12 +445,7 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
                                 (hipStream_t)hip_stream));
     if (in_kernel) {
         *flagged = 1;
-    } else if (want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0 && plan.args.head + plan.args.tail == 0 &&
-               g_policy.load(std::memory_order_relaxed) == POL_STREAM) {
-        // Only when every result store of the launch is a write-through vector store: those are in
-        // memory when the reduction kernel ends.  Peeled head/tail elements (and everything under the
-        // default cache policy) may still sit dirty in an L2 until the runtime's own release at a
-        // stream synchronisation, so such launches keep completing through the stream.
+    } else if (tail_ok) {
         hipLaunchKernelGGL(tail_flag_kernel, dim3(1), dim3(1), 0, (hipStream_t)hip_stream, dev_flag, seq);
         if (hipGetLastError() == hipSuccess) {
             *flagged = 1; // otherwise the caller waits for the stream, which still works
