@@ -315,16 +315,19 @@ def test_datagen_matches_oracle_generator(rocm, oracle, dt):
 
 
 def test_completion_word_threshold_and_sequences(rocm, oracle):
-    """Small launches complete through a host-mapped word the kernel writes,
-    large ones through the stream.  Sizes on both sides of the switch (8192
-    workgroups of 512 floats here), grids that fill the 64 arrival-counter
-    shards unevenly (65, 100, 129, 1000 workgroups), many back-to-back blocking
-    calls (sequence numbers advance per pooled event), results checked every
-    time."""
+    """Completion through a host-mapped word: written by the launch itself
+    (up to 1024 workgroups of 512 floats here, up to 8192 when the result has
+    peeled head/tail elements), by a one-lane kernel queued behind a larger
+    launch without such elements, and not at all beyond (then the stream is
+    waited for).  Sizes on every side of those switches, grids that fill the
+    64 arrival-counter shards unevenly (65, 100, 129, 1000 workgroups), many
+    back-to-back blocking calls (sequence numbers advance per pooled event),
+    results checked every time."""
     dt, op = Dt.FLOAT32, Op.SUM
     tile = 512
-    for size in (1, 63, 64 * tile, 65 * tile, 100 * tile + 3, 129 * tile - 1, 1000 * tile + 17, 8192 * tile - 1,
-                 8192 * tile, 8192 * tile + 1, 8193 * tile + 5):
+    for size in (1, 63, 64 * tile, 65 * tile, 100 * tile + 3, 129 * tile - 1, 1000 * tile + 17, 1024 * tile,
+                 1025 * tile, 2048 * tile + 4, 8192 * tile - 1, 8192 * tile, 8192 * tile + 1, 8193 * tile + 5,
+                 20000 * tile):
         c = Case(dt, size, 1)
         try:
             c.fill_random(oracle, 21)
