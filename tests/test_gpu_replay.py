@@ -208,6 +208,47 @@ def test_large_vectors_stream_ordered_overlap(rocm, oracle):
         rk.close()
 
 
+def test_four_threads_run_collectives_at_once(rocm):
+    """test/test_mt.c: 4 threads, each with a team of its own, run allreduce
+    after allreduce (INT32 SUM, count 32, the closed form of test_mt.c:58) --
+    here each thread drives its own set of loopback ranks through the one
+    component.  Together they want more pooled events than the component has,
+    so transport marks fall back to stream waits and reductions to the
+    blocking entry now and then; every result must still be right."""
+    import threading
+    P, iters = 6, 12
+    expect = [P * (P + 1) // 2 + P * (i + 12345) for i in range(32)]
+    teams = [Ranks(_kat(P)) for _ in range(4)]
+    errors = []
+
+    def worker(t):
+        rk = teams[t]
+        try:
+            for it in range(iters):
+                alg = ALLREDUCE[(t + it) % 2]
+                st, _ = rocm.replay_run(alg, rk.src_ptrs(), rk.dst_ptrs(), 32, Dt.INT32, Op.SUM, radix=2 + (t + it) % 3,
+                                        stream_ordered=bool((t + it // 2) % 2))
+                if st != Status.OK:
+                    errors.append((t, it, alg, "status", st))
+                    return
+                for r in range(P):
+                    if rk.result(r).tolist() != expect:
+                        errors.append((t, it, alg, "rank", r))
+                        return
+        except Exception as e:      # noqa: BLE001 -- reported by the main thread
+            errors.append((t, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(100)
+    assert not any(th.is_alive() for th in threads), "a thread is stuck"
+    assert errors == []
+    for rk in teams:
+        rk.close()
+
+
 def test_c_program_in_the_shape_of_the_reference_tests():
     """tests/c/test_rocm_allreduce.c: a C program laid out like
     test/test_mpi_cuda_allreduce.c and test/test_mpi_cuda_reduce.c, driving the

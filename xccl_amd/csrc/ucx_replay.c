@@ -406,6 +406,7 @@ static xccl_status_t issue_reduce(ctx_t *c, rank_state_t *s, void *s1, void *s2,
                                   size_t stride)
 {
     const xccl_replay_params_t *p = c->p;
+    xccl_status_t               st;
 
     if (n2 == 0) {
         c->stats->reduce_calls++;
@@ -428,9 +429,16 @@ static xccl_status_t issue_reduce(ctx_t *c, rank_state_t *s, void *s1, void *s2,
     if (count == 0) {
         return XCCL_OK; /* nothing to launch, nothing to wait for */
     }
-    return n2 == 0 ? xccl_mem_component_reduce_nb(s1, s2, out, count, p->dtype, p->op, MT, NULL, &s->reduce_ev)
-                   : xccl_mem_component_reduce_multi_nb(s1, s2, out, n2, count, stride, p->dtype, p->op, MT, NULL,
-                                                        &s->reduce_ev);
+    st = n2 == 0 ? xccl_mem_component_reduce_nb(s1, s2, out, count, p->dtype, p->op, MT, NULL, &s->reduce_ev)
+                 : xccl_mem_component_reduce_multi_nb(s1, s2, out, n2, count, stride, p->dtype, p->op, MT, NULL,
+                                                      &s->reduce_ev);
+    if (st == XCCL_ERR_NO_RESOURCE) {
+        /* the component's event pool is empty (other collectives hold it): this reduction blocks */
+        s->reduce_ev = NULL;
+        st = n2 == 0 ? xccl_mem_component_reduce(s1, s2, out, count, p->dtype, p->op, MT)
+                     : xccl_mem_component_reduce_multi(s1, s2, out, n2, count, stride, p->dtype, p->op, MT);
+    }
+    return st;
 }
 
 /* The "reduce in flight" phase: XCCL_OK once the result may be read. */
