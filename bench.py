@@ -128,6 +128,17 @@ def latency_sweep(mc, hip, iters, full):
                 row[mode] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
                              "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
             res["n%d_%dB" % (nsrc, b)] = row
+    # blocking calls from several host threads at once (XCCL_THREAD_MODE_MULTIPLE, reference test/test_mt.c):
+    # 4 sources x 1 KiB, every thread on operands of its own
+    tb = hip.DeviceBuffer(8 * 8192)
+    for th in (1, 2, 4):
+        st, ns = mc.bench_latency_mt(th, 8192, tb.ptr, tb.ptr + 1024, tb.ptr + 4096, 3, 256, 1024, Dt.FLOAT32, Op.SUM,
+                                     iters)
+        assert st == Status.OK
+        ns = ns[:, iters // 10:]
+        res["threads%d_n4_1024B" % th] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
+                                          "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
+    tb.close()
     # the memory-type probe libxccl issues at least twice per collective (mem_component.c:150-174)
     host = np.zeros(16, dtype=np.uint8)
     for name, ptr in (("device", buf.ptr), ("unregistered_host", host.ctypes.data)):
@@ -416,7 +427,7 @@ def main():
             os.makedirs(a.out_dir, exist_ok=True)
             json.dump(lat, open(os.path.join(a.out_dir, "latency.json"), "w"), indent=1)
             out["latency_us"] = {k: v for k, v in lat.items()
-                                 if k.endswith(("_4B", "_1024B", "_32768B")) or k.startswith(("mem_type", "alloc_free"))}
+                                 if k.endswith(("_4B", "_1024B", "_32768B")) or k.startswith(("mem_type", "alloc_free", "threads"))}
         else:
             out["latency_us"] = lat
 

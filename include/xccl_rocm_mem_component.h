@@ -99,8 +99,14 @@ extern "C" {
  *
  * reduce_nb / reduce_multi_nb: same arithmetic contract as reduce /
  * reduce_multi, but the call returns once the kernel is enqueued.
- *   stream == NULL : enqueue on the component's own stream (the one the
- *                    synchronous entries use), so successive calls are
+ *   stream == NULL : enqueue on the component's stream of the CALLING THREAD
+ *                    (the one the synchronous entries use on that thread), so
+ *                    successive calls of one thread are ordered among
+ *                    themselves.  Threads are spread round-robin over up to 4
+ *                    streams per device (XCCL_MC_ROCM_THREAD_STREAMS, 1..4),
+ *                    so that blocking calls of several threads
+ *                    (XCCL_THREAD_MODE_MULTIPLE) do not queue up behind each
+ *                    other's kernels; calls of different threads are not
  *                    ordered among themselves;
  *   stream != NULL : enqueue on *(hipStream_t*)stream->stream.
  *   event  != NULL : *event receives a pooled event recorded right after the
@@ -127,8 +133,9 @@ typedef struct xccl_rocm_mem_component {
                                      xccl_stream_t *stream,
                                      xccl_mc_event_t **event);
     xccl_status_t (*event_wait)(xccl_mc_event_t *event);
-    /* hipStream_t of the component for the current device (created on first
-     * use), as void*.  For callers that time or order work against it. */
+    /* The component's hipStream_t for the calling thread on the current
+     * device (created on first use), as void*.  For callers that time or
+     * order work against it. */
     xccl_status_t (*get_stream)(void **hip_stream);
 } xccl_rocm_mem_component_t;
 

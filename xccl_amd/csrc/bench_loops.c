@@ -207,3 +207,66 @@ xccl_status_t xccl_rocm_bench_region_time(xccl_rocm_mem_component_t *mc, void *s
     }
     return XCCL_OK;
 }
+
+/*
+ * `threads` host threads (at most 16) call the blocking reduce_multi entry at
+ * the same time, `iters` times each, every thread on operands of its own
+ * (thread t uses sbuf1 + t * thread_pitch and so on); ns_out receives
+ * threads * iters per-call durations, thread after thread.  What a
+ * XCCL_THREAD_MODE_MULTIPLE application sees (reference test/test_mt.c).
+ */
+#include <pthread.h>
+
+typedef struct {
+    xccl_rocm_mem_component_t *mc;
+    char                      *s1, *s2, *out;
+    size_t                     count, size, stride, iters;
+    xccl_dt_t                  dtype;
+    xccl_op_t                  op;
+    uint64_t                  *ns;
+    xccl_status_t              st;
+} mt_arg_t;
+
+static void *mt_worker(void *p)
+{
+    mt_arg_t *a = (mt_arg_t *)p;
+    size_t    i;
+
+    for (i = 0; i < a->iters && a->st == XCCL_OK; i++) {
+        const uint64_t t0 = now_ns();
+        a->st    = a->mc->super.reduce_multi(a->s1, a->s2, a->out, a->count, a->size, a->stride, a->dtype, a->op);
+        a->ns[i] = now_ns() - t0;
+    }
+    return NULL;
+}
+
+xccl_status_t xccl_rocm_bench_latency_mt(xccl_rocm_mem_component_t *mc, int threads, size_t thread_pitch, void *sbuf1,
+                                         void *sbuf2, void *rbuf, size_t count, size_t size, size_t stride,
+                                         xccl_dt_t dtype, xccl_op_t op, size_t iters, uint64_t *ns_out)
+{
+    pthread_t th[16];
+    mt_arg_t  arg[16];
+    int       t;
+
+    if (threads < 1 || threads > 16) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    for (t = 0; t < threads; t++) {
+        arg[t] = (mt_arg_t){mc, (char *)sbuf1 + t * thread_pitch, (char *)sbuf2 + t * thread_pitch,
+                            (char *)rbuf + t * thread_pitch, count, size, stride, iters, dtype, op,
+                            ns_out + (size_t)t * iters, XCCL_OK};
+        if (pthread_create(&th[t], NULL, mt_worker, &arg[t]) != 0) {
+            threads = t;
+            break;
+        }
+    }
+    for (t = 0; t < threads; t++) {
+        pthread_join(th[t], NULL);
+    }
+    for (t = 0; t < threads; t++) {
+        if (arg[t].st != XCCL_OK) {
+            return arg[t].st;
+        }
+    }
+    return XCCL_OK;
+}

@@ -39,6 +39,12 @@
 
 #define MC_MAX_DEVICES 64
 
+/* Reduction streams per device.  Every calling thread sticks to one of them
+ * (assigned round-robin on its first call), so that blocking calls from
+ * several threads (XCCL_THREAD_MODE_MULTIPLE) do not queue up behind each
+ * other's kernels; 4 = the hardware queues a process gets by default. */
+#define MC_NUM_STREAMS 4
+
 /* Synchronous reductions of at most this many bytes per vector are launched
  * through the graph path (XCCL_MC_ROCM_GRAPH_MAX_BYTES overrides; 0 = never). */
 #define MC_DEFAULT_GRAPH_MAX_BYTES 0
@@ -92,8 +98,7 @@ typedef struct mc_rocm_stream_request {
 
 typedef struct mc_rocm_device {
     atomic_int               ready; /* 0 = untouched, 1 = usable */
-    hipStream_t              stream;      /* reductions */
-    hipStream_t              gate_stream; /* stream gates: a gate must never sit in front of a reduction */
+    hipStream_t              stream[MC_NUM_STREAMS]; /* reductions: one per calling thread, round-robin */
     int                     *gate_words;  /* pinned, mapped */
     uint32_t                *flag_words; /* pinned, mapped: completion words of the events */
     uint32_t                *arrival_counts; /* device */
@@ -104,6 +109,7 @@ typedef struct mc_rocm_device {
 static mc_rocm_device_t mc_devices[MC_MAX_DEVICES];
 static pthread_mutex_t  mc_init_lock = PTHREAD_MUTEX_INITIALIZER;
 static size_t           mc_graph_max_bytes;
+static int              mc_num_streams = MC_NUM_STREAMS; /* XCCL_MC_ROCM_THREAD_STREAMS, 1 .. MC_NUM_STREAMS */
 static uint64_t         mc_gate_timeout_ns;
 
 #define MC_HIP(call)                                                              \
@@ -157,6 +163,10 @@ static void mc_rocm_read_config(void)
     if (s != NULL) {
         mc_gate_timeout_ns = strtoull(s, NULL, 0) * 1000000ull;
     }
+    s = getenv("XCCL_MC_ROCM_THREAD_STREAMS");
+    if (s != NULL && atoi(s) >= 1 && atoi(s) <= MC_NUM_STREAMS) {
+        mc_num_streams = atoi(s);
+    }
     s = getenv("XCCL_MC_ROCM_POOL_MAX_BYTES");
     if (s != NULL) {
         pool_limit = (size_t)strtoull(s, NULL, 0);
@@ -196,11 +206,10 @@ static void mc_rocm_device_destroy(mc_rocm_device_t *d)
     if (d->arrival_counts != NULL) {
         (void)hipFree(d->arrival_counts);
     }
-    if (d->gate_stream != NULL) {
-        (void)hipStreamDestroy(d->gate_stream);
-    }
-    if (d->stream != NULL) {
-        (void)hipStreamDestroy(d->stream);
+    for (i = 0; i < MC_NUM_STREAMS; i++) {
+        if (d->stream[i] != NULL) {
+            (void)hipStreamDestroy(d->stream[i]);
+        }
     }
     memset(d, 0, sizeof(*d));
 }
@@ -210,8 +219,7 @@ static xccl_status_t mc_rocm_device_create_parts(mc_rocm_device_t *d)
 {
     int i;
 
-    MC_HIP(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
-    MC_HIP(hipStreamCreateWithFlags(&d->gate_stream, hipStreamNonBlocking));
+    MC_HIP(hipStreamCreateWithFlags(&d->stream[0], hipStreamNonBlocking));
     MC_HIP(hipHostMalloc((void **)&d->gate_words,
                          XCCL_ROCM_MC_NUM_STREAM_REQUESTS * sizeof(int),
                          hipHostMallocMapped));
@@ -230,8 +238,8 @@ static xccl_status_t mc_rocm_device_create_parts(mc_rocm_device_t *d)
     MC_HIP(hipMalloc((void **)&d->arrival_counts,
                      XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_DONE_COUNT_BYTES));
     MC_HIP(hipMemsetAsync(d->arrival_counts, 0,
-                          XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_DONE_COUNT_BYTES, d->stream));
-    MC_HIP(hipStreamSynchronize(d->stream));
+                          XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_DONE_COUNT_BYTES, d->stream[0]));
+    MC_HIP(hipStreamSynchronize(d->stream[0]));
     for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
         mc_rocm_event_t *ev = &d->events[i];
         MC_HIP(hipEventCreateWithFlags(&ev->hip_event, hipEventDisableTiming));
@@ -281,6 +289,35 @@ static xccl_status_t mc_rocm_device(mc_rocm_device_t **out)
         pthread_mutex_unlock(&mc_init_lock);
     }
     *out = d;
+    return st;
+}
+
+/* The reduction stream of the calling thread on this device: every thread
+ * sticks to one of mc_num_streams streams, handed out round-robin at its first
+ * call; streams beyond the first are created when a thread first needs one. */
+static xccl_status_t mc_rocm_thread_stream(mc_rocm_device_t *d, hipStream_t *out)
+{
+    static atomic_uint       next_slot;
+    static _Thread_local int slot = -1;
+    xccl_status_t            st = XCCL_OK;
+
+    if (slot < 0) {
+        slot = (int)(atomic_fetch_add(&next_slot, 1) % (unsigned)mc_num_streams);
+    }
+    if (__atomic_load_n(&d->stream[slot], __ATOMIC_ACQUIRE) == NULL) {
+        pthread_mutex_lock(&mc_init_lock);
+        if (d->stream[slot] == NULL) {
+            hipStream_t hs = NULL;
+            if (hipStreamCreateWithFlags(&hs, hipStreamNonBlocking) != hipSuccess) {
+                (void)hipGetLastError();
+                st = XCCL_ERR_NO_MESSAGE;
+            } else {
+                __atomic_store_n(&d->stream[slot], hs, __ATOMIC_RELEASE);
+            }
+        }
+        pthread_mutex_unlock(&mc_init_lock);
+    }
+    *out = d->stream[slot];
     return st;
 }
 
@@ -438,7 +475,10 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
     if (st != XCCL_OK) {
         return st;
     }
-    hs = d->stream;
+    st = mc_rocm_thread_stream(d, &hs);
+    if (st != XCCL_OK) {
+        return st;
+    }
     if (stream != NULL) {
         st = mc_rocm_user_stream(stream, &hs);
         if (st != XCCL_OK) {
@@ -631,11 +671,15 @@ static xccl_status_t mc_rocm_event_free(xccl_mc_event_t *event)
 }
 
 /* cuda_mem_component.c:139-162: block the USER's stream until the host calls
- * finish_stream_activity.  A gate kernel polls a host-mapped word; the user
- * stream waits on an event recorded behind it.  Gates run on a stream of their
- * own: the reference puts its spin kernel on the stream its reductions use,
- * so a reduction issued while a gate is shut would wait for the very
- * collective that is waiting for the reduction. */
+ * finish_stream_activity.  A gate kernel that polls a host-mapped word goes
+ * straight into the user's stream.  The reference puts its spin kernel on the
+ * stream its reductions use and lets the user's stream wait for an event behind
+ * it: a reduction issued while the gate is shut then waits for the very
+ * collective that is waiting for the reduction, gates of different user
+ * streams wait for each other, and two hardware queues are held up instead of
+ * one.  (Streams that share the user's hardware queue -- a process has 4 by
+ * default -- are still held up while a gate is shut; the gate's wait is
+ * bounded.) */
 static xccl_status_t
 mc_rocm_start_stream_activity(xccl_stream_t *stream,
                               xccl_mem_component_stream_request_t **req)
@@ -670,13 +714,12 @@ mc_rocm_start_stream_activity(xccl_stream_t *stream,
         return XCCL_ERR_NO_RESOURCE;
     }
     __atomic_store_n(r->flag, 0, __ATOMIC_RELEASE);
-    st = xccl_rocm_stream_gate(r->dev_flag, mc_gate_timeout_ns, d->gate_stream);
+    st = xccl_rocm_stream_gate(r->dev_flag, mc_gate_timeout_ns, user);
     if (st != XCCL_OK) {
         atomic_store(&r->is_free, MC_SLOT_FREE);
         return st;
     }
-    if (hipEventRecord(r->hip_event, d->gate_stream) != hipSuccess ||
-        hipStreamWaitEvent(user, r->hip_event, 0) != hipSuccess) {
+    if (hipEventRecord(r->hip_event, user) != hipSuccess) { /* tells when the gate kernel has retired */
         /* open the gate again: nothing may stay blocked behind a failure */
         __atomic_store_n(r->flag, 1, __ATOMIC_RELEASE);
         atomic_store(&r->is_free, MC_SLOT_FREE);
@@ -712,7 +755,10 @@ static xccl_status_t mc_rocm_get_stream(void **hip_stream)
     if (st != XCCL_OK) {
         return st;
     }
-    *hip_stream = (void *)d->stream;
+    st = mc_rocm_thread_stream(d, (hipStream_t *)hip_stream);
+    if (st != XCCL_OK) {
+        return st;
+    }
     return XCCL_OK;
 }
 
@@ -742,8 +788,16 @@ static void mc_rocm_close(void)
         for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS; i++) {
             __atomic_store_n(d->requests[i].flag, 1, __ATOMIC_RELEASE); /* open any gate left shut */
         }
-        (void)hipStreamSynchronize(d->gate_stream);
-        (void)hipStreamSynchronize(d->stream);
+        for (i = 0; i < XCCL_ROCM_MC_NUM_STREAM_REQUESTS; i++) {
+            if (atomic_load(&d->requests[i].is_free) != MC_SLOT_FREE) {
+                (void)hipEventSynchronize(d->requests[i].hip_event); /* its gate kernel has left the queue */
+            }
+        }
+        for (i = 0; i < MC_NUM_STREAMS; i++) {
+            if (d->stream[i] != NULL) {
+                (void)hipStreamSynchronize(d->stream[i]);
+            }
+        }
         xccl_rocm_graph_cache_destroy();
         mc_rocm_device_destroy(d); /* also clears `ready` */
     }

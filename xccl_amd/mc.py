@@ -149,6 +149,7 @@ def benchkit_lib():
         lib.xccl_rocm_bench_latency.argtypes = [_vp, _vp, _int, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
         lib.xccl_rocm_bench_kernel_times.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp]
         lib.xccl_rocm_bench_region_time.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp, _vp]
+        lib.xccl_rocm_bench_latency_mt.argtypes = [_vp, _int, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
         lib.xccl_rocm_bench_mem_type.argtypes = [_vp, _vp, _sz, _vp, _vp]
         lib.xccl_rocm_bench_alloc_free.argtypes = [_vp, _sz, _sz, _vp]
         _datagen_lib = lib
@@ -325,6 +326,16 @@ def bench_region_time(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters:
     hip.event_destroy(e0)
     hip.event_destroy(e1)
     return _st(st), ms.value
+
+
+def bench_latency_mt(threads: int, thread_pitch: int, sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters: int):
+    """Per-call durations in ns, shape (threads, iters), of blocking reduce_multi calls
+    issued by `threads` host threads at once, thread t on operands t * thread_pitch further on."""
+    import numpy as np
+    out = np.zeros((threads, iters), dtype=np.uint64)
+    st = benchkit_lib().xccl_rocm_bench_latency_mt(_c.addressof(component()), threads, thread_pitch, sbuf1, sbuf2, rbuf,
+                                                   count, size, stride, int(dtype), int(op), iters, out.ctypes.data)
+    return _st(st), out
 
 
 def bench_mem_type(ptr, iters: int):
