@@ -17,6 +17,9 @@
  *     src/team_lib/ucx/xccl_ucx_lib.c:631-632);
  *   - events are created once (the reference re-creates one on every record,
  *     cuda_mem_component.c:220, and leaks the old one);
+ *   - calling threads are spread over up to four reduction streams, and a
+ *     stream gate goes into the user's stream, not in front of reductions;
+ *   - freed device blocks are cached for the next mem_alloc (mc_pool.h);
  *   - small launches report completion through a host-mapped word the kernel
  *     writes itself, which the host sees sooner than the queue's signal;
  *   - the vtable is extended with stream-ordered reductions whose completion
