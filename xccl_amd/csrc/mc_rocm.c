@@ -298,15 +298,22 @@ static xccl_status_t mc_rocm_device(mc_rocm_device_t **out)
 /* The reduction stream of the calling thread on this device: every thread
  * sticks to one of mc_num_streams streams, handed out round-robin at its first
  * call; streams beyond the first are created when a thread first needs one. */
+static unsigned mc_rocm_thread_index(void)
+{
+    static atomic_uint       next_index;
+    static _Thread_local int index = -1;
+
+    if (index < 0) {
+        index = (int)(atomic_fetch_add(&next_index, 1) & 0x7fffffffu);
+    }
+    return (unsigned)index;
+}
+
 static xccl_status_t mc_rocm_thread_stream(mc_rocm_device_t *d, hipStream_t *out)
 {
-    static atomic_uint       next_slot;
-    static _Thread_local int slot = -1;
-    xccl_status_t            st = XCCL_OK;
+    const int     slot = (int)(mc_rocm_thread_index() % (unsigned)mc_num_streams);
+    xccl_status_t st   = XCCL_OK;
 
-    if (slot < 0) {
-        slot = (int)(atomic_fetch_add(&next_slot, 1) % (unsigned)mc_num_streams);
-    }
     if (__atomic_load_n(&d->stream[slot], __ATOMIC_ACQUIRE) == NULL) {
         pthread_mutex_lock(&mc_init_lock);
         if (d->stream[slot] == NULL) {
@@ -397,10 +404,13 @@ static xccl_status_t mc_rocm_mem_type(void *ptr, ucs_memory_type_t *mem_type)
 
 static mc_rocm_event_t *mc_rocm_claim_event(mc_rocm_device_t *d)
 {
-    int i, expect;
+    /* threads start their search in different quarters of the pool, so that
+     * they do not all fight for the first slots */
+    const unsigned first = (mc_rocm_thread_index() % 4u) * (XCCL_ROCM_MC_NUM_EVENTS / 4u);
+    int            i, expect;
 
     for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
-        mc_rocm_event_t *ev = &d->events[i];
+        mc_rocm_event_t *ev = &d->events[(first + (unsigned)i) % XCCL_ROCM_MC_NUM_EVENTS];
         expect = MC_SLOT_FREE;
         if (!atomic_compare_exchange_strong(&ev->is_free, &expect, MC_SLOT_BUSY)) {
             continue;
