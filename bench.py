@@ -139,6 +139,17 @@ def latency_sweep(mc, hip, iters, full):
         res["threads%d_n4_1024B" % th] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
                                           "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
     tb.close()
+    # memcpy_async + event_record + event_query: one message of the loopback transport / one mpod alltoall step
+    ms = mc.Stream(hip.stream_create())
+    cb = hip.DeviceBuffer(2 << 20)
+    for nb in (1024, 65536, 1 << 20):
+        st, ns = mc.bench_memcpy(ms, cb.ptr, cb.ptr + (1 << 20), nb, 1000)
+        assert st == Status.OK
+        res["memcpy_event_%dB" % nb] = {"p50": round(float(np.percentile(ns[100:], 50)) / 1e3, 2),
+                                        "p99": round(float(np.percentile(ns[100:], 99)) / 1e3, 2)}
+    hip.stream_synchronize(ms.hip_stream)
+    hip.stream_destroy(ms.hip_stream)
+    cb.close()
     # the memory-type probe libxccl issues at least twice per collective (mem_component.c:150-174)
     host = np.zeros(16, dtype=np.uint8)
     for name, ptr in (("device", buf.ptr), ("unregistered_host", host.ctypes.data)):
@@ -427,7 +438,7 @@ def main():
             os.makedirs(a.out_dir, exist_ok=True)
             json.dump(lat, open(os.path.join(a.out_dir, "latency.json"), "w"), indent=1)
             out["latency_us"] = {k: v for k, v in lat.items()
-                                 if k.endswith(("_4B", "_1024B", "_32768B")) or k.startswith(("mem_type", "alloc_free", "threads"))}
+                                 if k.endswith(("_4B", "_1024B", "_32768B")) or k.startswith(("mem_type", "alloc_free", "threads", "memcpy"))}
         else:
             out["latency_us"] = lat
 

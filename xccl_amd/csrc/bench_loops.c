@@ -270,3 +270,37 @@ xccl_status_t xccl_rocm_bench_latency_mt(xccl_rocm_mem_component_t *mc, int thre
     }
     return XCCL_OK;
 }
+
+/*
+ * Times `iters` rounds of memcpy_async(src -> dst, len) on `xs` followed by
+ * event_record and event_query polling until done -- one message of the
+ * loopback transport, or one step of the mpod team library's alltoall
+ * (reference src/team_lib/mpod/xccl_mpod_alltoall.c:41-163 uses the
+ * same three entries).
+ */
+xccl_status_t xccl_rocm_bench_memcpy(xccl_rocm_mem_component_t *mc, xccl_stream_t *xs, void *src, void *dst, size_t len,
+                                     size_t iters, uint64_t *ns_out)
+{
+    size_t i;
+
+    for (i = 0; i < iters; i++) {
+        xccl_mc_event_t *ev = NULL;
+        const uint64_t   t0 = now_ns();
+        xccl_status_t    st = mc->super.memcpy_async(src, dst, len, xs);
+        if (st != XCCL_OK) {
+            return st;
+        }
+        st = mc->super.event_record(xs, &ev);
+        if (st != XCCL_OK) {
+            return st;
+        }
+        while ((st = mc->super.event_query(ev)) == XCCL_INPROGRESS) {
+        }
+        mc->super.event_free(ev);
+        ns_out[i] = now_ns() - t0;
+        if (st != XCCL_OK) {
+            return st;
+        }
+    }
+    return XCCL_OK;
+}

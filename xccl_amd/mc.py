@@ -150,6 +150,7 @@ def benchkit_lib():
         lib.xccl_rocm_bench_kernel_times.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp]
         lib.xccl_rocm_bench_region_time.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp, _vp]
         lib.xccl_rocm_bench_latency_mt.argtypes = [_vp, _int, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
+        lib.xccl_rocm_bench_memcpy.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _vp]
         lib.xccl_rocm_bench_mem_type.argtypes = [_vp, _vp, _sz, _vp, _vp]
         lib.xccl_rocm_bench_alloc_free.argtypes = [_vp, _sz, _sz, _vp]
         _datagen_lib = lib
@@ -335,6 +336,15 @@ def bench_latency_mt(threads: int, thread_pitch: int, sbuf1, sbuf2, rbuf, count,
     out = np.zeros((threads, iters), dtype=np.uint64)
     st = benchkit_lib().xccl_rocm_bench_latency_mt(_c.addressof(component()), threads, thread_pitch, sbuf1, sbuf2, rbuf,
                                                    count, size, stride, int(dtype), int(op), iters, out.ctypes.data)
+    return _st(st), out
+
+
+def bench_memcpy(stream: Stream, src, dst, nbytes: int, iters: int):
+    """Durations in ns of `iters` rounds of memcpy_async + event_record + event_query polling."""
+    import numpy as np
+    out = np.zeros(iters, dtype=np.uint64)
+    st = benchkit_lib().xccl_rocm_bench_memcpy(_c.addressof(component()), stream.ref(), src, dst, nbytes, iters,
+                                               out.ctypes.data)
     return _st(st), out
 
 
