@@ -69,7 +69,7 @@ xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf,
  * a one-lane kernel is queued that stores the word, provided every result
  * store of that launch is a write-through vector store (no peeled head or
  * tail elements: 16-byte-aligned operands and a byte count that is a multiple
- * of 16; streaming cache policy); launches that are not keep counting up to
+ * of 16); launches that are not keep counting up to
  * 8192 workgroups.  Beyond that, or with XCCL_MC_ROCM_TAIL_FLAG=0 in the
  * environment where the queued kernel would be used, or if its launch
  * fails, `*flagged` is 0 and the caller waits for the stream as usual.  One launch at a time per (count, flag) pair.  No
@@ -84,6 +84,25 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
                                              uint32_t *dev_flag, uint32_t seq,
                                              int *flagged);
 
+/*
+ * xccl_rocm_reduce_multi_flagged for callers that must not allocate: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  The arrival counters
+ * live in a static device array inside the library (XCCL_ROCM_DONE_COUNT_BYTES
+ * per GPU, held until the process ends) instead of coming from the caller, and
+ * the call allocates nothing: it enqueues one small kernel that clears the
+ * counters and the reduction itself, which always counts its own workgroups
+ * and stores `seq` to `*dev_flag` (caller-owned, device-visible) when the last
+ * one is through.  Limit: at most 8192 workgroups, i.e. 8 MiB per vector; a
+ * larger call returns XCCL_ERR_INVALID_PARAM and prints why.  Every call on a
+ * GPU shares that GPU's array: calls that overlap in time on one GPU race.
+ */
+xccl_status_t xccl_rocm_reduce_multi_flagged_static(void *sbuf1, void *sbuf2, void *rbuf,
+                                                    size_t count, size_t size,
+                                                    size_t stride, xccl_dt_t dtype,
+                                                    xccl_op_t op, void *hip_stream,
+                                                    uint32_t *dev_flag, uint32_t seq);
+
 /* Same contract and same kernel as xccl_rocm_reduce_multi_impl, but enqueued
  * as one launch of a pre-instantiated single-kernel-node hipGraph whose node
  * parameters are patched per call (a small per-device cache keeps the most
@@ -95,6 +114,20 @@ xccl_status_t xccl_rocm_reduce_multi_graph(void *sbuf1, void *sbuf2, void *rbuf,
                                            size_t stride, xccl_dt_t dtype,
                                            xccl_op_t op, void *hip_stream);
 
+/* The graph launch with the completion word of xccl_rocm_reduce_multi_flagged
+ * (launches of up to 8192 workgroups; `*flagged` tells) and, for measurement,
+ * the host time of its steps in `ns_parts` (may be NULL; 4 values:
+ * planning, lock + slot search, building or patching the graph,
+ * hipGraphLaunch).  The sequence number is a kernel argument, so a flagged
+ * launch patches its node on every call. */
+xccl_status_t xccl_rocm_reduce_multi_graph_flagged(void *sbuf1, void *sbuf2, void *rbuf,
+                                                   size_t count, size_t size,
+                                                   size_t stride, xccl_dt_t dtype,
+                                                   xccl_op_t op, void *hip_stream,
+                                                   uint32_t *dev_count,
+                                                   uint32_t *dev_flag, uint32_t seq,
+                                                   int *flagged, uint64_t *ns_parts);
+
 /* Drop every cached graph of the current device (component close). */
 void xccl_rocm_graph_cache_destroy(void);
 
@@ -102,18 +135,15 @@ void xccl_rocm_graph_cache_destroy(void);
  * Launch-shape knobs, for measurement.  `blocks_per_cu` caps the grid at
  * blocks_per_cu x (compute units) workgroups of one wavefront; beyond the cap
  * workgroups loop over tiles.  0 restores the built-in default (a cap large
- * enough that every tile gets its own workgroup).  `cache_policy`: 1 =
- * streaming accesses (non-temporal loads, system-scope stores; the default),
- * 0 = default-policy loads and stores.  `resident_per_cu`: how many
- * workgroups may be resident on a compute unit at once (enforced by asking
- * for LDS the kernel never touches); 0 = the built-in choice by source count
- * (8 to 12), 32 or more = no limit.  All are process-global and may also be
+ * enough that every tile gets its own workgroup).  `resident_per_cu`: how
+ * many workgroups may be resident on a compute unit at once (enforced by
+ * asking for LDS the kernel never touches); 0 = the built-in choice by source
+ * count (16 to 32), 32 or more = no limit, 1 and 2 behave as 3 (a workgroup
+ * cannot ask for more than 64 KiB).  Both are process-global and may also be
  * set through the environment (XCCL_MC_ROCM_BLOCKS_PER_CU,
- * XCCL_MC_ROCM_CACHE_POLICY, XCCL_MC_ROCM_RESIDENT_PER_CU), read once at
- * first launch.
+ * XCCL_MC_ROCM_RESIDENT_PER_CU), read once at first launch.
  */
-void xccl_rocm_set_launch_shape(int blocks_per_cu, int cache_policy,
-                                int resident_per_cu);
+void xccl_rocm_set_launch_shape(int blocks_per_cu, int resident_per_cu);
 
 /* What a launch with these arguments would be: grid/block size and the
  * mangled kernel name (truncated into `name`, if not NULL).  Host-only apart

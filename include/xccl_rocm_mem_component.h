@@ -117,7 +117,20 @@ extern "C" {
  * With event == NULL the entries do nothing but enqueue one kernel, so a
  * caller may record them into its own hipGraph through stream capture; an
  * event must not be requested while capturing (its completion is tied to
- * this one launch, not to later replays).
+ * this one launch, not to later replays).  The component creates its
+ * per-device resources on the first call on a device, which allocates and
+ * synchronises: make that call outside any capture (a call with a capturing
+ * `stream` on a device not yet used returns XCCL_ERR_NO_RESOURCE).
+ *
+ * finish_stream_activity returns XCCL_ERR_NO_PROGRESS when the gate kernel
+ * had already given up (XCCL_MC_ROCM_GATE_TIMEOUT_MS, default 30 s; the
+ * reference kernel spins without a bound): work queued behind the gate then
+ * ran before the collective finished, and the caller must not trust stream
+ * order for it.
+ *
+ * mem_free keeps the block for the next mem_alloc and does not wait for the
+ * device (the reference's cudaFree does): free a block only after all work
+ * that touches it has completed.
  * These replace the launch + cudaStreamSynchronize pair of the reference
  * (xccl_cuda_reduce_multi.cu:42-44,140) at the call sites named above.
  */

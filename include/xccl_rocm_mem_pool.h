@@ -11,9 +11,11 @@
  * allocation plus a runtime free that waits for the device.  The component
  * keeps freed blocks by size class (request rounded up to 4 KiB at least, then
  * to an eighth-of-a-power-of-two step: at most 12.5 % over-allocation) and
- * hands them out again.  A block returned by mem_free is reusable at once:
- * as with any allocator, the caller frees only memory no queued work still
- * uses.
+ * hands them out again.  A block returned by mem_free is reusable at once,
+ * and -- unlike the reference's cudaFree -- mem_free does not wait for the
+ * device: free a block only after every stream-ordered reduction, copy or
+ * kernel that touches it has completed (event_query / event_wait say when),
+ * or another thread's mem_alloc may receive it while that work still runs.
  *
  * The limit is the number of bytes that may sit in FREE blocks; least recently
  * freed blocks are released first.  Default 8 GiB, or the environment variable

@@ -200,20 +200,22 @@ def test_source_counts(rocm, oracle, n2):
 def test_grid_cap_and_ragged_tiles(rocm, oracle):
     """Sizes that leave a partial tile, with the grid capped low (1 and 64
     workgroups per compute unit) so that every workgroup loops over tiles, then
-    the other cache policy without a residency cap."""
+    residency caps at both ends of the range (3 workgroups per compute unit,
+    which also exercises the clamp of the LDS request, and no cap)."""
     lib = rocm.component_lib()
     try:
         for bpc in (1, 64):
-            lib.xccl_rocm_set_launch_shape(bpc, 1, 0)
+            lib.xccl_rocm_set_launch_shape(bpc, 0)
             for size in (256 * 4 * 2 * 256 + 13, 1 << 20, (1 << 20) + 4 * 255 + 3):
                 run_and_check(rocm, oracle, Dt.FLOAT32, Op.SUM, size, 7, seed=9, check_untouched=False)
                 run_and_check(rocm, oracle, Dt.INT8, Op.SUM, size, 2, seed=9, check_untouched=False)
-        lib.xccl_rocm_set_launch_shape(0, 0, 32)   # default-policy loads and stores, no residency cap
-        for dt, op in ((Dt.FLOAT32, Op.SUM), (Dt.INT16, Op.MAX), (Dt.FLOAT64, Op.MIN)):
-            run_and_check(rocm, oracle, dt, op, (1 << 18) + 77, 7, seed=10)
-            run_and_check(rocm, oracle, dt, op, 1001, 4, off1=dt_size(dt), seed=10)
+        for resident in (1, 3, 32):
+            lib.xccl_rocm_set_launch_shape(0, resident)
+            for dt, op in ((Dt.FLOAT32, Op.SUM), (Dt.INT16, Op.MAX), (Dt.FLOAT64, Op.MIN)):
+                run_and_check(rocm, oracle, dt, op, (1 << 20) + 77, 7, seed=10, check_untouched=False)
+                run_and_check(rocm, oracle, dt, op, 1001, 4, off1=dt_size(dt), seed=10)
     finally:
-        lib.xccl_rocm_set_launch_shape(0, 1, 0)
+        lib.xccl_rocm_set_launch_shape(0, 0)
 
 
 def test_randomised_shapes(rocm, oracle):

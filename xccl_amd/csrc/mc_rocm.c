@@ -295,6 +295,24 @@ static xccl_status_t mc_rocm_device(mc_rocm_device_t **out)
     return st;
 }
 
+/* The current device's resources for work that goes into the caller's stream.
+ * Creating them allocates and synchronises, which would invalidate a capture
+ * in progress: a first call on a device must not come from inside one. */
+static xccl_status_t mc_rocm_device_for_stream(mc_rocm_device_t **out, hipStream_t hs)
+{
+    int                    dev = 0;
+    hipStreamCaptureStatus cs  = hipStreamCaptureStatusNone;
+
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < MC_MAX_DEVICES &&
+        atomic_load_explicit(&mc_devices[dev].ready, memory_order_acquire) == 0 &&
+        hipStreamIsCapturing(hs, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) {
+        fprintf(stderr, "xccl mc_rocm: first use of device %d inside a stream capture; call any entry of the "
+                        "component once outside the capture first\n", dev);
+        return XCCL_ERR_NO_RESOURCE;
+    }
+    return mc_rocm_device(out);
+}
+
 /* The reduction stream of the calling thread on this device: every thread
  * sticks to one of mc_num_streams streams, handed out round-robin at its first
  * call; streams beyond the first are created when a thread first needs one. */
@@ -347,6 +365,10 @@ static xccl_status_t mc_rocm_mem_alloc(void **ptr, size_t len)
     return XCCL_OK;
 }
 
+/* The block goes back to the cache, not to the runtime, so the implicit device
+ * synchronisation of the reference's cudaFree (cuda_mem_component.c:40-44) is
+ * gone: free a block only after all work that touches it has completed, or the
+ * next mem_alloc may hand it out while that work still runs. */
 static xccl_status_t mc_rocm_mem_free(void *ptr)
 {
     int rc;
@@ -484,19 +506,20 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
     if (st != XCCL_OK) {
         return st;
     }
-    st = mc_rocm_device(&d);
-    if (st != XCCL_OK) {
-        return st;
-    }
-    st = mc_rocm_thread_stream(d, &hs);
-    if (st != XCCL_OK) {
-        return st;
-    }
     if (stream != NULL) {
         st = mc_rocm_user_stream(stream, &hs);
         if (st != XCCL_OK) {
             return st;
         }
+        st = mc_rocm_device_for_stream(&d, hs);
+    } else {
+        st = mc_rocm_device(&d);
+        if (st == XCCL_OK) {
+            st = mc_rocm_thread_stream(d, &hs);
+        }
+    }
+    if (st != XCCL_OK) {
+        return st;
     }
     if (event != NULL || want_sync) {
         /* a pooled event brings the completion word; a blocking call can do
@@ -747,16 +770,25 @@ static xccl_status_t
 mc_rocm_finish_stream_activity(xccl_mem_component_stream_request_t *req)
 {
     mc_rocm_stream_request_t *r;
+    int                       old;
 
     if (req == NULL) {
         return XCCL_ERR_INVALID_PARAM;
     }
     r = (mc_rocm_stream_request_t *)((char *)req -
                                      offsetof(mc_rocm_stream_request_t, super));
-    __atomic_store_n(r->flag, 1, __ATOMIC_RELEASE);
+    old = __atomic_exchange_n(r->flag, 1, __ATOMIC_ACQ_REL);
     /* Not reusable until its gate kernel has seen the word and left the
      * queue; start_stream_activity checks that when it claims the slot. */
     atomic_store(&r->is_free, MC_SLOT_DRAINING);
+    if (old == 2) {
+        /* the gate kernel ran into its time limit and let the user's stream go
+         * on before the collective had finished: stream order was not kept */
+        fprintf(stderr, "xccl mc_rocm: stream gate gave up after %llu ms (XCCL_MC_ROCM_GATE_TIMEOUT_MS) before "
+                        "finish_stream_activity; work queued behind it ran early\n",
+                (unsigned long long)(mc_gate_timeout_ns / 1000000ull));
+        return XCCL_ERR_NO_PROGRESS;
+    }
     return XCCL_OK;
 }
 

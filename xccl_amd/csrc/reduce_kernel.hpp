@@ -7,18 +7,26 @@
 //     rbuf[i] = acc
 // The reference's CUDA kernel (xccl_cuda_reduce_multi.cu:17-40) keeps acc in
 // global memory and reads 2/4/8 bytes per lane; here every lane moves 16 bytes
-// per source with one global_load_dwordx4, all sources of a tile are in flight
-// before the first fold, and acc never leaves registers.
+// per source with one buffer_load_dwordx4 and acc never leaves registers.
 //
-// Shape, from measurement on MI355X (fp32 SUM, 8 x 256 MiB): one-wave
-// workgroups, one tile per workgroup (a grid as large as the tile count; the
-// grid-stride loop only runs when that exceeds the grid cap) beat 256-lane
-// persistent workgroups by ~25%; streaming cache policy (non-temporal loads,
-// system-scope write-through stores) beats default-policy accesses by ~17%;
-// holding the workgroups resident per compute unit to about ten (the launch
-// asks for LDS it never touches) adds 4-12%: the memory side is saturated
-// long before the wave slots are, and fewer waves in flight keep the
-// addresses being served close together.
+// Shape, from measurement on MI355X.  A workgroup is one wavefront and owns
+// one tile: 64 x 16 bytes = 1 KiB of every source.  The wave walks the
+// sources in fold order with two loads in flight (ping-pong registers):
+// while source j is folded into the accumulator, sources j+1 and j+2 are on
+// their way.  One kernel serves any number of sources.  The obvious
+// alternative -- issue the loads of all sources at the same offset at once,
+// then fold -- makes every wave send a burst of same-offset requests to
+// vectors that lie a power of two apart, which land on the same memory
+// channels at the same moment: on the headline shape (8 x 256 MiB, fp32 SUM)
+// that is 6.4 TB/s against 6.8-7.0 TB/s for the source-by-source walk, and
+// 5.5 against 6.6 TB/s with 1 GiB vectors.  Persistent workgroups that loop
+// over tiles, larger tiles and multi-wave workgroups all measured slower.
+// Sources are read once: non-temporal loads.  The result is about to be read
+// by another agent (the NIC sending it, the next round's kernel): stores carry
+// system scope (sc0 sc1), i.e. write through instead of lingering dirty in L2.
+// The launch asks for LDS it never touches to hold the resident workgroups
+// per compute unit to 16-32 (by source count): the memory side saturates
+// before the wave slots do.
 //
 // Layout of one call, in elements of T:
 //     [0, head)                 peeled so that the vector body starts on a
@@ -28,8 +36,9 @@
 //     [.., .. + tail)           fewer than VE elements
 // Head and tail are folded element-wise by the first lanes of the last block.
 // Vector accesses are emitted as dwordx4 whatever the address is (the device
-// runs in unaligned access mode), so a source whose alignment differs from
-// the peeled one costs extra cache-line touches, never correctness.
+// runs in unaligned access mode, for buffer instructions too), so a source
+// whose alignment differs from the peeled one costs extra cache-line touches,
+// never correctness.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -108,48 +117,31 @@ template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBand>(u32x4 a, u32
 template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBor>(u32x4 a, u32x4 b)  { return a | b; }
 template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBxor>(u32x4 a, u32x4 b) { return a ^ b; }
 
-// Cache policy of the vector accesses.
-//   POL_PLAIN   default loads and stores.
-//   POL_STREAM  sources are read once: non-temporal loads.  The result is
-//               about to be read by another agent (the NIC sending it, the
-//               next round's kernel): stores carry system scope (sc0 sc1),
-//               i.e. write through instead of lingering dirty in L2.
-enum { POL_PLAIN = 0, POL_STREAM = 1 };
+// Vector accesses go through buffer instructions: the descriptor (scalar
+// registers) holds the tile's base address and its length in bytes, the lane
+// supplies a 32-bit offset.  The hardware drops stores and returns zero for
+// loads beyond the length, so the ragged last tile needs no branch, and the
+// cache-policy bits are ordinary operands the compiler tracks (no inline asm).
+//   loads:  nt            (aux bit 1)
+//   stores: sc0 sc1       (aux bits 0 and 4)
+constexpr int kAuxLoad  = 0x02;
+constexpr int kAuxStore = 0x11;
+// DST_SEL_X/Y/Z/W = X/Y/Z/W, 32-bit data format: the raw-buffer descriptor word gfx9 expects
+constexpr int kRsrcFlags = 0x00027000;
 
-// Vector accesses are addressed as (uniform 64-bit base) + (32-bit lane
-// offset): the base lives in scalar registers, one VGPR serves every access of
-// a tile, and a wave gets from its first instruction to its first load in a
-// few cycles -- with one tile per wave, the prologue is part of every tile.
-template <int POL>
-__device__ __forceinline__ u32x4 vload(const char *base, uint32_t off)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const char *base, uint32_t bytes)
 {
-    if (POL == POL_STREAM) {
-        return __builtin_nontemporal_load((const u32x4_u *)(base + off));
-    }
-    return *(const u32x4_u *)(base + off);
+    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)bytes, kRsrcFlags);
 }
 
-template <int POL>
-__device__ __forceinline__ void vstore(char *base, uint32_t off, u32x4 v)
+__device__ __forceinline__ u32x4 vload(__amdgpu_buffer_rsrc_t r, uint32_t off)
 {
-    if (POL == POL_STREAM) {
-        // No builtin emits a 16-byte store with these scope bits, hence asm --
-        // and asm the compiler's hazard recogniser cannot see into, so the
-        // statement has to be hazard-free by construction:
-        //  * it takes its address as a 64-bit VGPR pair, never a scalar base:
-        //    a VMEM instruction that reads an SGPR within 5 wait states of a
-        //    VALU write to it (v_readlane restoring a spilled SGPR does that)
-        //    sees the old value, i.e. a wild address;
-        //  * it ends in s_nop: gfx9 reads the data registers of a store wider
-        //    than 8 bytes one cycle after issue, and a VALU write to them in
-        //    the next slot corrupts the stored value.
-        // A store has no result register, so the compiler's s_waitcnt
-        // bookkeeping stays valid; the clobber keeps it ordered after the loads.
-        char *p = base + off;
-        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
-    } else {
-        *(u32x4_u *)(base + off) = v;
-    }
+    return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, kAuxLoad);
+}
+
+__device__ __forceinline__ void vstore(__amdgpu_buffer_rsrc_t r, uint32_t off, u32x4 v)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)off, 0, kAuxStore);
 }
 
 template <typename T>
@@ -172,98 +164,48 @@ __device__ __forceinline__ void fold_element(const ReduceArgs &a, ptrdiff_t rel)
     __builtin_memcpy(a.dst + rel, &acc, sizeof(T));
 }
 
-// One tile = UNROLL x kBlock vectors; lane t of the block owns vectors
-// v0 + u*kBlock + t.  NSRC > 0: exactly NSRC sources, all NSRC*UNROLL loads
-// issued before the first fold.  NSRC == 0: any number of sources, loaded four
-// at a time.  GUARD: the tile may run past nvec.
-template <typename T, class Op, int NSRC, int UNROLL, int POL, bool GUARD>
+// One tile: kBlock vectors, lane t owns vector v0 + t.  Sources are walked in
+// fold order, two loads in flight.  The scheduling barriers pin the issue
+// order: left alone, the compiler hoists and clusters the loads and the walk
+// turns back into a burst.
+template <typename T, class Op>
 __device__ __forceinline__ void fold_tile(const ReduceArgs &a, size_t v0)
 {
-    const size_t tile_off = v0 * 16; // uniform: same for every lane of the workgroup
-    const char  *p1       = a.s1 + tile_off;
-    const char  *p2       = a.s2 + tile_off;
-    char        *pd       = a.dst + tile_off;
-    uint32_t     off[UNROLL];
-    bool         live[UNROLL];
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-        off[u]  = (uint32_t)(u * kBlock + (int)threadIdx.x) * 16u;
-        live[u] = !GUARD || v0 + (size_t)u * kBlock + threadIdx.x < a.nvec;
-    }
+    const size_t   left  = a.nvec - v0;
+    const uint32_t bytes = (uint32_t)(left < (size_t)kBlock ? left : (size_t)kBlock) * 16u; // the descriptor clips the ragged tile
+    const size_t   toff  = v0 * 16; // uniform: same for every lane of the workgroup
+    const uint32_t off   = threadIdx.x * 16u;
+    const uint32_t n2    = a.n2;
+    const char    *p     = a.s2 + toff; // vector j of sbuf2 as the walk advances
 
-    if constexpr (NSRC > 0) {
-        constexpr int N = NSRC;
-        u32x4         r[UNROLL][N];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            if (live[u]) {
-                r[u][0] = vload<POL>(p1, off[u]);
-#pragma unroll
-                for (int j = 1; j < N; ++j) {
-                    r[u][j] = vload<POL>(p2 + (size_t)(j - 1) * a.stride, off[u]);
-                }
-            }
+    // A load past the last source gets a descriptor of length zero: the
+    // hardware returns zeros without touching memory, and the walk needs no
+    // branch around a load (a branch there makes the compiler wait for every
+    // load in flight where the paths join).
+    u32x4 acc = vload(tile_rsrc(a.s1 + toff, bytes), off);
+    u32x4 l0  = vload(tile_rsrc(p, bytes), off);
+    p += a.stride;
+    u32x4 l1 = vload(tile_rsrc(p, n2 > 1 ? bytes : 0), off);
+    __builtin_amdgcn_sched_barrier(0);
+    acc = vfold<T, Op>(acc, l0); // OP(sbuf1, sbuf2{0})
+    __builtin_amdgcn_sched_barrier(0);
+    // here: l1 holds vector j of sbuf2 (in flight), p points at it, l0 is free
+    for (uint32_t j = 1; j < n2; j += 2) {
+        p += a.stride;
+        l0 = vload(tile_rsrc(p, j + 1 < n2 ? bytes : 0), off);
+        __builtin_amdgcn_sched_barrier(0);
+        acc = vfold<T, Op>(l1, acc); // OP(sbuf2{j}, acc)
+        __builtin_amdgcn_sched_barrier(0);
+        if (j + 1 >= n2) {
+            break;
         }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            if (live[u]) {
-                u32x4 acc = vfold<T, Op>(r[u][0], r[u][1]);
-#pragma unroll
-                for (int j = 2; j < N; ++j) {
-                    acc = vfold<T, Op>(r[u][j], acc);
-                }
-                vstore<POL>(pd, off[u], acc);
-            }
-        }
-    } else {
-        u32x4 acc[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            if (live[u]) {
-                u32x4 x = vload<POL>(p1, off[u]);
-                u32x4 y = vload<POL>(p2, off[u]);
-                acc[u]  = vfold<T, Op>(x, y);
-            }
-        }
-        uint32_t j = 1;
-        for (; j + 4 <= a.n2; j += 4) {
-            const char *p = p2 + (size_t)j * a.stride;
-            u32x4       r[UNROLL][4];
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                if (live[u]) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        r[u][k] = vload<POL>(p + (size_t)k * a.stride, off[u]);
-                    }
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                if (live[u]) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        acc[u] = vfold<T, Op>(r[u][k], acc[u]);
-                    }
-                }
-            }
-        }
-        for (; j < a.n2; ++j) {
-            const char *p = p2 + (size_t)j * a.stride;
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                if (live[u]) {
-                    acc[u] = vfold<T, Op>(vload<POL>(p, off[u]), acc[u]);
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            if (live[u]) {
-                vstore<POL>(pd, off[u], acc[u]);
-            }
-        }
+        p += a.stride;
+        l1 = vload(tile_rsrc(p, j + 2 < n2 ? bytes : 0), off);
+        __builtin_amdgcn_sched_barrier(0);
+        acc = vfold<T, Op>(l0, acc);
+        __builtin_amdgcn_sched_barrier(0);
     }
+    vstore(tile_rsrc(a.dst + toff, bytes), off, acc);
 }
 
 // Tells the host that the launch is complete without going through the queue's
@@ -271,21 +213,20 @@ __device__ __forceinline__ void fold_tile(const ReduceArgs &a, size_t v0)
 // part).  Every workgroup -- one wave -- waits until its own result stores have
 // completed, then counts itself in; the last one to arrive publishes the
 // sequence number and re-arms the counter.
-//   Streaming policy: the vector stores are system-scope write-through, so
-//   "completed" already means "in memory"; a wave only needs its vmcnt to
-//   drain (a workgroup-scope release) before it counts itself in.  Stores made
-//   with default policy (`wrote_plain`: the element-wise head/tail, or every
-//   store under POL_PLAIN) sit dirty in this XCD's L2 and need the wave's own
-//   system-scope release, which writes that L2 back.
+//   The vector stores are system-scope write-through, so "completed" already
+//   means "in memory": the wave waits for its outstanding memory operations
+//   (s_waitcnt vmcnt(0)) before it counts itself in.  Neither a workgroup-scope
+//   fence nor the relaxed arrival atomic would make it wait.  Stores made with
+//   default policy (`wrote_plain`: the element-wise head/tail) sit dirty in this
+//   XCD's L2 and need the wave's own system-scope release, which writes that L2
+//   back and waits as well.
 // One contended atomic per workgroup: for small grids only.
-template <int POL>
 __device__ __forceinline__ void publish_completion(const ReduceArgs &a, bool wrote_plain)
 {
-    if (POL != POL_STREAM || wrote_plain) {
+    if (wrote_plain) {
         __threadfence_system();
-    } else {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if (threadIdx.x == 0) {
         // Arrival counting in two levels, so that no single word takes more than
         // grid/kDoneShards increments: workgroup b counts into shard b % shards, the
@@ -310,24 +251,10 @@ __device__ __forceinline__ void publish_completion(const ReduceArgs &a, bool wro
     }
 }
 
-template <typename T, class Op, int NSRC, int UNROLL, int POL>
+template <typename T, class Op>
 __global__ void __launch_bounds__(kBlock) reduce_multi_kernel(const ReduceArgs a)
 {
-    constexpr size_t tile = (size_t)kBlock * UNROLL;
-    const size_t     step = (size_t)gridDim.x * tile;
-    size_t           v0   = (size_t)blockIdx.x * tile;
-
-    // Fetch the completion-word pointer together with the other arguments: left
-    // alone, its scalar load sinks below the stores and the wave waits for it
-    // there instead of retiring.
-    uint32_t *const done_flag = a.done_flag;
-    asm volatile("" : : "s"(done_flag));
-
-    // Head and tail first: they use ordinary loads and stores, whose completion
-    // the compiler tracks.  The tiles end in asm stores it cannot see; anything
-    // it had to order after them (a loop back-edge, say) would make it wait for
-    // every outstanding store, and the wave would sit on its slot for a
-    // write-through round trip instead of retiring.
+    // Head and tail: ordinary element-wise loads and stores, by the last workgroup.
     const bool edges = blockIdx.x == gridDim.x - 1 && a.head + a.tail != 0;
     if (edges) {
         const size_t t = threadIdx.x;
@@ -337,70 +264,29 @@ __global__ void __launch_bounds__(kBlock) reduce_multi_kernel(const ReduceArgs a
             fold_element<T, Op>(a, (ptrdiff_t)(a.nvec * 16 + (t - a.head) * sizeof(T)));
         }
     }
-    if (step >= a.nvec) {
-        // the usual launch: at most one tile per workgroup, straight-line code
-        if (v0 < a.nvec) {
-            if (v0 + tile <= a.nvec) {
-                fold_tile<T, Op, NSRC, UNROLL, POL, false>(a, v0);
-            } else {
-                fold_tile<T, Op, NSRC, UNROLL, POL, true>(a, v0);
-            }
-        }
-    } else {
-        // more tiles than the grid cap allows workgroups: loop
-        for (; v0 < a.nvec; v0 += step) {
-            if (v0 + tile <= a.nvec) {
-                fold_tile<T, Op, NSRC, UNROLL, POL, false>(a, v0);
-            } else {
-                fold_tile<T, Op, NSRC, UNROLL, POL, true>(a, v0);
-            }
-        }
+    // One tile per workgroup in the usual launch; the loop only runs on when
+    // there are more tiles than the grid cap allows workgroups.
+    const size_t step = (size_t)gridDim.x * kBlock;
+    for (size_t v0 = (size_t)blockIdx.x * kBlock; v0 < a.nvec; v0 += step) {
+        fold_tile<T, Op>(a, v0);
     }
-    if (done_flag != nullptr) {
-        publish_completion<POL>(a, edges);
+    if (a.done_flag != nullptr) {
+        publish_completion(a, edges);
     }
 }
 
 // ---- table of instantiations ---------------------------------------------
-// Source-count variants: exact counts for the radices the k-nomial and
-// scatter-reduce steps use (2, 3, 4, 8, 16 sources), and the any-count kernel.
-enum { NV_ANY = 0, NV_2, NV_3, NV_4, NV_8, NV_16, NV_COUNT };
-
-constexpr int nsrc_of(int nv) { return nv == NV_2 ? 2 : nv == NV_3 ? 3 : nv == NV_4 ? 4 : nv == NV_8 ? 8 : nv == NV_16 ? 16 : 0; }
-// vectors per lane per tile: two -- with the resident-workgroup cap, two tiles
-// per wave measured best for 2, 4, 8 and 16 sources alike -- except 16 sources
-// of 8-bit elements, where 32 vectors in flight plus the unpacked bytes do not
-// fit the register file and the compiler would spill to scratch memory
-constexpr int unroll_of(int nv, int esize) { return (nv == NV_16 && esize == 1) ? 1 : 2; }
-
 struct KernelEntry {
-    const void *fn[2][NV_COUNT]; // [cache policy][variant]
-    int         elem_size;       // sizeof(T) the kernel folds in
+    const void *fn;        // reduce_multi_kernel<T, Op>
+    int         elem_size; // sizeof(T) the kernel folds in
 };
-
-template <typename T, class Op, int POL, int NV>
-constexpr const void *kernel_ptr()
-{
-    return (const void *)&reduce_multi_kernel<T, Op, nsrc_of(NV), unroll_of(NV, (int)sizeof(T)), POL>;
-}
 
 template <typename T, class Op>
 KernelEntry make_entry()
 {
     KernelEntry e;
-    e.fn[0][NV_ANY] = kernel_ptr<T, Op, POL_PLAIN, NV_ANY>();
-    e.fn[0][NV_2]   = kernel_ptr<T, Op, POL_PLAIN, NV_2>();
-    e.fn[0][NV_3]   = kernel_ptr<T, Op, POL_PLAIN, NV_3>();
-    e.fn[0][NV_4]   = kernel_ptr<T, Op, POL_PLAIN, NV_4>();
-    e.fn[0][NV_8]   = kernel_ptr<T, Op, POL_PLAIN, NV_8>();
-    e.fn[0][NV_16]  = kernel_ptr<T, Op, POL_PLAIN, NV_16>();
-    e.fn[1][NV_ANY] = kernel_ptr<T, Op, POL_STREAM, NV_ANY>();
-    e.fn[1][NV_2]   = kernel_ptr<T, Op, POL_STREAM, NV_2>();
-    e.fn[1][NV_3]   = kernel_ptr<T, Op, POL_STREAM, NV_3>();
-    e.fn[1][NV_4]   = kernel_ptr<T, Op, POL_STREAM, NV_4>();
-    e.fn[1][NV_8]   = kernel_ptr<T, Op, POL_STREAM, NV_8>();
-    e.fn[1][NV_16]  = kernel_ptr<T, Op, POL_STREAM, NV_16>();
-    e.elem_size     = (int)sizeof(T);
+    e.fn        = (const void *)&reduce_multi_kernel<T, Op>;
+    e.elem_size = (int)sizeof(T);
     return e;
 }
 

@@ -9,6 +9,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 namespace xccl_rocm {
 namespace {
@@ -20,9 +21,11 @@ constexpr int kDefaultBlocksPerCu = 8192;
 
 // Resident one-wave workgroups per compute unit for large launches, by source
 // count (0 = these defaults, > 0 = this many for every call, >= kNoResidentCap =
-// no cap).  Measured optimum on MI355X: 12 for 2-3 sources, 10 up to 8, 8 beyond.
+// no cap).  Measured on MI355X with the source-by-source walk: no cap for 2
+// sources, 16 for 3-4, 24 beyond.
 constexpr int    kNoResidentCap = 32;
 constexpr size_t kLdsPerCu      = 160 * 1024;
+constexpr size_t kLdsPerGroup   = 64 * 1024; // most a workgroup may ask for
 
 // Launches of at most this many workgroups may count their own arrivals for a
 // completion word: each workgroup pays an atomic on one of 64 shared counters
@@ -32,9 +35,9 @@ constexpr size_t kLdsPerCu      = 160 * 1024;
 constexpr unsigned kMaxFlaggedGrid = 8192;
 
 std::atomic<int> g_blocks_per_cu{-1}; // -1: not read from the environment yet
-std::atomic<int> g_policy{-1};
 std::atomic<int> g_resident{0};
 std::atomic<int> g_tail_flag{1};
+std::atomic<unsigned> g_shape_epoch{0}; // bumped when a launch-shape knob changes
 std::atomic<unsigned> g_max_counted_grid{1024}; // measured: counting wins up to ~512 workgroups, ties at 2048, loses 3-5 % at 8192
 std::atomic<int> g_cu_count[kMaxDevices];
 
@@ -43,7 +46,6 @@ void read_env_once()
     if (g_blocks_per_cu.load(std::memory_order_acquire) >= 0) {
         return;
     }
-    const char *pol = getenv("XCCL_MC_ROCM_CACHE_POLICY");
     const char *bpc = getenv("XCCL_MC_ROCM_BLOCKS_PER_CU");
     const char *res = getenv("XCCL_MC_ROCM_RESIDENT_PER_CU");
     const char *tf  = getenv("XCCL_MC_ROCM_TAIL_FLAG");
@@ -54,7 +56,6 @@ void read_env_once()
     }
     int         v   = bpc ? atoi(bpc) : 0;
     g_resident.store(res && atoi(res) > 0 ? atoi(res) : 0, std::memory_order_release);
-    g_policy.store((pol && atoi(pol) == POL_PLAIN) ? POL_PLAIN : POL_STREAM, std::memory_order_release);
     g_blocks_per_cu.store(v > 0 ? v : kDefaultBlocksPerCu, std::memory_order_release);
 }
 
@@ -144,12 +145,13 @@ unsigned lds_for_resident(uint32_t nsrc, size_t grid, int cus)
 {
     int cap = g_resident.load(std::memory_order_relaxed);
     if (cap == 0) {
-        cap = nsrc <= 3 ? 12 : nsrc <= 8 ? 10 : 8;
+        cap = nsrc <= 2 ? kNoResidentCap : nsrc <= 4 ? 16 : 24;
     }
     if (cap >= kNoResidentCap || grid <= (size_t)cap * (size_t)cus) {
         return 0; // the whole grid is resident at once anyway
     }
-    return (unsigned)((kLdsPerCu / (size_t)cap) & ~(size_t)511);
+    size_t lds = (kLdsPerCu / (size_t)cap) & ~(size_t)511;
+    return (unsigned)(lds > kLdsPerGroup ? kLdsPerGroup : lds); // 1 or 2 asked for: 2.5 is the fewest LDS can enforce
 }
 
 bool same_plan(const Plan &a, const Plan &b)
@@ -210,7 +212,6 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     const size_t   ve    = 16 / esize;
     const uint32_t n2    = count == 0 ? 1u : (uint32_t)count;
     const uint32_t nsrc  = n2 + 1;
-    const int      nv    = nsrc == 2 ? NV_2 : nsrc == 3 ? NV_3 : nsrc == 4 ? NV_4 : nsrc == 8 ? NV_8 : nsrc == 16 ? NV_16 : NV_ANY;
 
     size_t head = pick_head_bytes(s1, s2, dst, stride, n2, esize) / esize;
     if (head > elems) {
@@ -229,7 +230,7 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     a.done_count = nullptr;
     a.done_flag  = nullptr;
 
-    const size_t tile  = (size_t)kBlock * unroll_of(nv, e->elem_size);
+    const size_t tile  = (size_t)kBlock;
     const size_t tiles = (a.nvec + tile - 1) / tile;
     const size_t cap   = (size_t)cus * (size_t)g_blocks_per_cu.load(std::memory_order_relaxed);
     size_t       grid  = tiles < cap ? tiles : cap;
@@ -238,8 +239,46 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     }
     plan->grid      = (unsigned)grid;
     plan->lds_bytes = lds_for_resident(nsrc, grid, cus);
-    plan->fn   = e->fn[g_policy.load(std::memory_order_relaxed) == POL_PLAIN ? POL_PLAIN : POL_STREAM][nv];
+    plan->fn        = e->fn;
     return XCCL_OK;
+}
+
+// The k-nomial and scatter-reduce rounds repeat identical calls (same buffers,
+// same shape) collective after collective; every thread keeps the plan of its
+// last call and skips kernel lookup, alignment vote and grid sizing when the
+// next call has the same arguments.
+struct PlanKey {
+    void     *s1, *s2, *dst;
+    size_t    count, size, stride;
+    int       dt, op;
+    unsigned  epoch;
+};
+
+struct PlanCache {
+    bool    valid = false;
+    PlanKey key;
+    Plan    plan;
+};
+
+thread_local PlanCache t_plan;
+
+xccl_status_t cached_plan(void *s1, void *s2, void *dst, size_t count, size_t size, size_t stride, xccl_dt_t dt,
+                          xccl_op_t op, Plan *plan)
+{
+    const unsigned epoch = g_shape_epoch.load(std::memory_order_acquire);
+    PlanCache     &c     = t_plan;
+    if (c.valid && c.key.s1 == s1 && c.key.s2 == s2 && c.key.dst == dst && c.key.count == count && c.key.size == size &&
+        c.key.stride == stride && c.key.dt == (int)dt && c.key.op == (int)op && c.key.epoch == epoch) {
+        *plan = c.plan;
+        return XCCL_OK;
+    }
+    xccl_status_t st = make_plan(s1, s2, dst, count, size, stride, dt, op, plan);
+    if (st == XCCL_OK) {
+        c.key   = PlanKey{s1, s2, dst, count, size, stride, (int)dt, (int)op, epoch};
+        c.plan  = *plan;
+        c.valid = true;
+    }
+    return st;
 }
 
 static_assert(XCCL_ROCM_DONE_COUNT_BYTES == (1 + kDoneShards) * kDoneStride * sizeof(uint32_t), "counter block size");
@@ -253,7 +292,8 @@ struct GraphSlot {
     hipGraph_t      graph = nullptr;
     hipGraphNode_t  node  = nullptr;
     hipGraphExec_t  exec  = nullptr;
-    hipEvent_t      done  = nullptr; // recorded after the last launch
+    hipStream_t     last_stream = nullptr; // where the last launch went
+    bool            last_stream_valid = false;
     uint64_t        stamp = 0;
 };
 
@@ -285,9 +325,6 @@ void destroy_slot(GraphSlot &s)
     if (s.graph) {
         (void)hipGraphDestroy(s.graph);
     }
-    if (s.done) {
-        (void)hipEventDestroy(s.done);
-    }
     s = GraphSlot();
 }
 
@@ -300,13 +337,25 @@ void destroy_slot(GraphSlot &s)
         }                                                                                          \
     } while (0)
 
-xccl_status_t graph_launch(Plan &plan, hipStream_t stream)
+uint64_t clock_ns()
+{
+    timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (uint64_t)ts.tv_sec * 1000000000ull + (uint64_t)ts.tv_nsec;
+}
+
+// Launches `plan` as a one-node graph: a slot whose instantiated graph has the
+// same arguments is replayed untouched, otherwise the least recently used slot
+// is patched.  `ns` (may be NULL) receives the host time of the three steps:
+// [0] lock + slot search, [1] building or patching the graph, [2] hipGraphLaunch.
+xccl_status_t graph_launch(Plan &plan, hipStream_t stream, uint64_t *ns)
 {
     int dev = 0;
     HIP_OR_FAIL(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) {
         return XCCL_ERR_NO_RESOURCE;
     }
+    uint64_t                    t = ns ? clock_ns() : 0;
     GraphCache                 &gc = g_graphs[dev];
     std::lock_guard<std::mutex> guard(gc.lock);
 
@@ -328,6 +377,11 @@ xccl_status_t graph_launch(Plan &plan, hipStream_t stream)
             }
         }
     }
+    if (ns) {
+        const uint64_t u = clock_ns();
+        ns[0] = u - t;
+        t     = u;
+    }
 
     if (hit == nullptr) {
         hipKernelNodeParams np;
@@ -337,8 +391,7 @@ xccl_status_t graph_launch(Plan &plan, hipStream_t stream)
             fill_node_params(&np, &victim->plan, argv);
             HIP_OR_FAIL(hipGraphCreate(&victim->graph, 0));
             if (hipGraphAddKernelNode(&victim->node, victim->graph, nullptr, 0, &np) != hipSuccess ||
-                hipGraphInstantiate(&victim->exec, victim->graph, nullptr, nullptr, 0) != hipSuccess ||
-                hipEventCreateWithFlags(&victim->done, hipEventDisableTiming) != hipSuccess) {
+                hipGraphInstantiate(&victim->exec, victim->graph, nullptr, nullptr, 0) != hipSuccess) {
                 destroy_slot(*victim);
                 (void)hipGetLastError();
                 return XCCL_ERR_NO_MESSAGE;
@@ -347,7 +400,9 @@ xccl_status_t graph_launch(Plan &plan, hipStream_t stream)
         } else {
             // The executable graph may still be running its previous launch
             // on another stream; patch it only once that launch has finished.
-            HIP_OR_FAIL(hipEventSynchronize(victim->done));
+            if (victim->last_stream_valid && victim->last_stream != stream) {
+                HIP_OR_FAIL(hipStreamSynchronize(victim->last_stream));
+            }
             victim->plan = plan;
             fill_node_params(&np, &victim->plan, argv);
             if (hipGraphExecKernelNodeSetParams(victim->exec, victim->node, &np) != hipSuccess) {
@@ -358,9 +413,18 @@ xccl_status_t graph_launch(Plan &plan, hipStream_t stream)
         }
         hit = victim;
     }
+    if (ns) {
+        const uint64_t u = clock_ns();
+        ns[1] = u - t;
+        t     = u;
+    }
     hit->stamp = ++gc.clock;
     HIP_OR_FAIL(hipGraphLaunch(hit->exec, stream));
-    HIP_OR_FAIL(hipEventRecord(hit->done, stream));
+    hit->last_stream       = stream;
+    hit->last_stream_valid = true;
+    if (ns) {
+        ns[2] = clock_ns() - t;
+    }
     return XCCL_OK;
 }
 
@@ -390,6 +454,60 @@ __global__ void stream_gate_kernel(int *flag, uint64_t max_ticks)
 
 using namespace xccl_rocm;
 
+namespace {
+
+// Plan of a call, or `*nothing` when there is nothing to launch (size == 0 is
+// a no-op for a supported pair, reference mem_component.c:129-131).
+xccl_status_t prepare(void *s1, void *s2, void *dst, size_t count, size_t size, size_t stride, xccl_dt_t dt,
+                      xccl_op_t op, Plan *plan, bool *nothing)
+{
+    *nothing = size == 0;
+    if (size == 0) {
+        return lookup(dt, op) ? XCCL_OK : XCCL_ERR_UNSUPPORTED;
+    }
+    return cached_plan(s1, s2, dst, count, size, stride, dt, op, plan);
+}
+
+// Arrival counters for xccl_rocm_reduce_multi_flagged_static: device memory that
+// exists from the moment the code object is loaded, so that entry never
+// allocates.  In host code the array's name is a stand-in, not a device
+// address: the address on each device comes from hipGetSymbolAddress, once per
+// device, and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) uint32_t scratch[XCCL_ROCM_DONE_COUNT_BYTES / sizeof(uint32_t)];
+
+std::atomic<uint32_t *> g_scratch_ptr[kMaxDevices];
+std::mutex              g_scratch_lock;
+
+xccl_status_t static_scratch(uint32_t **out)
+{
+    int dev = 0;
+    HIP_OR_FAIL(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) {
+        return XCCL_ERR_NO_RESOURCE;
+    }
+    uint32_t *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        std::lock_guard<std::mutex> guard(g_scratch_lock);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (p == nullptr) {
+            HIP_OR_FAIL(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return XCCL_OK;
+}
+
+// Clears the arrival counters (a fill kernel, not hipMemsetAsync: callers may be capturing).
+__global__ void clear_words_kernel(uint32_t *p, uint32_t n)
+{
+    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+        p[i] = 0;
+    }
+}
+
+} // namespace
+
 extern "C" {
 
 xccl_status_t xccl_rocm_reduce_supported(xccl_dt_t dtype, xccl_op_t op)
@@ -411,28 +529,21 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
     if (flagged) {
         *flagged = 0;
     }
-    if (lookup(dtype, op) == nullptr) {
-        return XCCL_ERR_UNSUPPORTED;
-    }
-    if (size == 0) {
-        return XCCL_OK;
-    }
     Plan          plan;
-    xccl_status_t st = make_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan);
-    if (st != XCCL_OK) {
+    bool          nothing = false;
+    xccl_status_t st      = prepare(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan, &nothing);
+    if (st != XCCL_OK || nothing) {
         return st;
     }
     // Who writes the completion word: the launch itself, counting its workgroups (cheapest for small
     // grids), or a one-lane kernel queued behind it (cheaper from about a thousand workgroups on).  The
     // second needs every result store of the launch to be a write-through vector store: those are in
-    // memory when the reduction kernel ends, while peeled head/tail elements (and everything under the
-    // default cache policy) may sit dirty in an L2 until the runtime's own release at a stream
-    // synchronisation -- such launches count up to the larger bound and beyond it complete through the
-    // stream.
+    // memory when the reduction kernel ends, while peeled head/tail elements may sit dirty in an L2 until
+    // the runtime's own release at a stream synchronisation -- such launches count up to the larger bound
+    // and beyond it complete through the stream.
     const bool     want_flag = dev_count != nullptr && dev_flag != nullptr && flagged != nullptr;
     const bool     tail_ok   = want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0 &&
-                               plan.args.head + plan.args.tail == 0 &&
-                               g_policy.load(std::memory_order_relaxed) == POL_STREAM;
+                               plan.args.head + plan.args.tail == 0;
     const unsigned counted   = tail_ok ? g_max_counted_grid.load(std::memory_order_relaxed) : kMaxFlaggedGrid;
     const bool     in_kernel = want_flag && plan.grid <= counted;
     if (in_kernel) {
@@ -454,6 +565,45 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
     return XCCL_OK;
 }
 
+xccl_status_t xccl_rocm_reduce_multi_flagged_static(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
+                                                    size_t stride, xccl_dt_t dtype, xccl_op_t op, void *hip_stream,
+                                                    uint32_t *dev_flag, uint32_t seq)
+{
+    if (dev_flag == nullptr) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    Plan          plan;
+    bool          nothing = false;
+    xccl_status_t st      = prepare(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan, &nothing);
+    if (st != XCCL_OK || nothing) {
+        return st;
+    }
+    if (plan.grid > kMaxFlaggedGrid) {
+        fprintf(stderr,
+                "xccl mc_rocm: xccl_rocm_reduce_multi_flagged_static takes at most %u KiB per vector (%u workgroups); "
+                "this call needs %u workgroups\n",
+                kMaxFlaggedGrid, kMaxFlaggedGrid, plan.grid);
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    uint32_t *counters = nullptr;
+    st = static_scratch(&counters);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    // The array keeps what the last call on this device left in it; a launch that
+    // ran to its end left zeros, one that did not may have left anything.
+    hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(256), 0, (hipStream_t)hip_stream, counters,
+                       (uint32_t)(XCCL_ROCM_DONE_COUNT_BYTES / sizeof(uint32_t)));
+    HIP_OR_FAIL(hipGetLastError());
+    plan.args.done_seq   = seq;
+    plan.args.done_count = counters;
+    plan.args.done_flag  = dev_flag;
+    void *argv[1] = {&plan.args};
+    HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, plan.lds_bytes,
+                                (hipStream_t)hip_stream));
+    return XCCL_OK;
+}
+
 xccl_status_t xccl_rocm_reduce_impl(void *sbuf1, void *sbuf2, void *target, size_t count, xccl_dt_t dtype,
                                     xccl_op_t op, void *hip_stream)
 {
@@ -463,18 +613,39 @@ xccl_status_t xccl_rocm_reduce_impl(void *sbuf1, void *sbuf2, void *target, size
 xccl_status_t xccl_rocm_reduce_multi_graph(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
                                            size_t stride, xccl_dt_t dtype, xccl_op_t op, void *hip_stream)
 {
-    if (lookup(dtype, op) == nullptr) {
-        return XCCL_ERR_UNSUPPORTED;
+    return xccl_rocm_reduce_multi_graph_flagged(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, hip_stream, nullptr,
+                                                nullptr, 0, nullptr, nullptr);
+}
+
+xccl_status_t xccl_rocm_reduce_multi_graph_flagged(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
+                                                   size_t stride, xccl_dt_t dtype, xccl_op_t op, void *hip_stream,
+                                                   uint32_t *dev_count, uint32_t *dev_flag, uint32_t seq,
+                                                   int *flagged, uint64_t *ns_parts)
+{
+    if (flagged) {
+        *flagged = 0;
     }
-    if (size == 0) {
-        return XCCL_OK;
-    }
-    Plan          plan;
-    xccl_status_t st = make_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan);
-    if (st != XCCL_OK) {
+    const uint64_t t0 = ns_parts ? clock_ns() : 0;
+    Plan           plan;
+    bool           nothing = false;
+    xccl_status_t  st      = prepare(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan, &nothing);
+    if (st != XCCL_OK || nothing) {
         return st;
     }
-    return graph_launch(plan, (hipStream_t)hip_stream);
+    if (dev_count != nullptr && dev_flag != nullptr && flagged != nullptr && plan.grid <= kMaxFlaggedGrid) {
+        plan.args.done_seq   = seq;
+        plan.args.done_count = dev_count;
+        plan.args.done_flag  = dev_flag;
+        *flagged             = 1;
+    }
+    if (ns_parts) {
+        ns_parts[0] = clock_ns() - t0; // planning
+    }
+    st = graph_launch(plan, (hipStream_t)hip_stream, ns_parts ? ns_parts + 1 : nullptr);
+    if (st != XCCL_OK && flagged) {
+        *flagged = 0;
+    }
+    return st;
 }
 
 void xccl_rocm_graph_cache_destroy(void)
@@ -487,19 +658,19 @@ void xccl_rocm_graph_cache_destroy(void)
     GraphCache                 &gc = g_graphs[dev];
     std::lock_guard<std::mutex> guard(gc.lock);
     for (GraphSlot &s : gc.slot) {
-        if (s.live) {
-            (void)hipEventSynchronize(s.done);
+        if (s.live && s.last_stream_valid) {
+            (void)hipStreamSynchronize(s.last_stream);
         }
         destroy_slot(s);
     }
 }
 
-void xccl_rocm_set_launch_shape(int blocks_per_cu, int cache_policy, int resident_per_cu)
+void xccl_rocm_set_launch_shape(int blocks_per_cu, int resident_per_cu)
 {
     read_env_once();
     g_resident.store(resident_per_cu > 0 ? resident_per_cu : 0, std::memory_order_release);
     g_blocks_per_cu.store(blocks_per_cu > 0 ? blocks_per_cu : kDefaultBlocksPerCu, std::memory_order_release);
-    g_policy.store(cache_policy == POL_PLAIN ? POL_PLAIN : POL_STREAM, std::memory_order_release);
+    g_shape_epoch.fetch_add(1, std::memory_order_release); // plans cached by the threads are stale now
 }
 
 xccl_status_t xccl_rocm_reduce_multi_plan(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,

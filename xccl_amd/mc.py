@@ -93,8 +93,15 @@ def component_lib():
         lib.xccl_rocm_reduce_multi_graph.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp]
         lib.xccl_rocm_graph_cache_destroy.argtypes = []
         lib.xccl_rocm_graph_cache_destroy.restype = None
-        lib.xccl_rocm_set_launch_shape.argtypes = [_int, _int, _int]
+        lib.xccl_rocm_set_launch_shape.argtypes = [_int, _int]
         lib.xccl_rocm_set_launch_shape.restype = None
+        _u32p = _c.POINTER(_c.c_uint32)
+        lib.xccl_rocm_reduce_multi_flagged.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp, _vp, _vp,
+                                                       _c.c_uint32, _c.POINTER(_int)]
+        lib.xccl_rocm_reduce_multi_flagged_static.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp, _vp,
+                                                              _c.c_uint32]
+        lib.xccl_rocm_reduce_multi_graph_flagged.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp, _vp, _vp,
+                                                             _c.c_uint32, _c.POINTER(_int), _c.POINTER(_c.c_uint64)]
         lib.xccl_rocm_reduce_multi_plan.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int,
                                                     _c.POINTER(_c.c_uint), _c.POINTER(_c.c_uint), _c.c_char_p, _sz]
         lib.xccl_rocm_stream_gate.argtypes = [_vp, _c.c_uint64, _vp]
