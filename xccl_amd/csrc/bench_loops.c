@@ -209,6 +209,45 @@ xccl_status_t xccl_rocm_bench_region_time(xccl_rocm_mem_component_t *mc, void *s
 }
 
 /*
+ * xccl_rocm_bench_region_time with the destination cycling through
+ * `rot_count` vectors `rot_pitch` bytes apart (launch i writes rbuf +
+ * (i % rot_count) * rot_pitch): a destination that is rewritten launch after
+ * launch partly stays in the memory-side cache, a rotating one does not.
+ */
+xccl_status_t xccl_rocm_bench_region_time_rot(xccl_rocm_mem_component_t *mc, void *sbuf1, void *sbuf2, void *rbuf,
+                                              size_t rot_count, size_t rot_pitch, size_t count, size_t size,
+                                              size_t stride, xccl_dt_t dtype, xccl_op_t op, size_t iters,
+                                              void *ev_begin, void *ev_end, float *ms_out)
+{
+    void         *stream = NULL;
+    xccl_status_t st     = mc->get_stream(&stream);
+    size_t        i;
+
+    if (st != XCCL_OK) {
+        return st;
+    }
+    if (rot_count == 0) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    if (hipEventRecord((hipEvent_t)ev_begin, (hipStream_t)stream) != hipSuccess) {
+        return XCCL_ERR_NO_MESSAGE;
+    }
+    for (i = 0; i < iters; i++) {
+        st = mc->reduce_multi_nb(sbuf1, sbuf2, (char *)rbuf + (i % rot_count) * rot_pitch, count, size, stride, dtype,
+                                 op, NULL, NULL);
+        if (st != XCCL_OK) {
+            return st;
+        }
+    }
+    if (hipEventRecord((hipEvent_t)ev_end, (hipStream_t)stream) != hipSuccess ||
+        hipStreamSynchronize((hipStream_t)stream) != hipSuccess ||
+        hipEventElapsedTime(ms_out, (hipEvent_t)ev_begin, (hipEvent_t)ev_end) != hipSuccess) {
+        return XCCL_ERR_NO_MESSAGE;
+    }
+    return XCCL_OK;
+}
+
+/*
  * `threads` host threads (at most 16) call the blocking reduce_multi entry at
  * the same time, `iters` times each, every thread on operands of its own
  * (thread t uses sbuf1 + t * thread_pitch and so on); ns_out receives
@@ -303,4 +342,66 @@ xccl_status_t xccl_rocm_bench_memcpy(xccl_rocm_mem_component_t *mc, xccl_stream_
         }
     }
     return XCCL_OK;
+}
+
+/*
+ * Where the time of a one-node graph launch goes.  Each of `iters` rounds
+ * issues one reduction through `graph_fn` (xccl_rocm_reduce_multi_graph_flagged)
+ * with a completion word, then polls the word's host view until the kernel has
+ * written it.  ns_out receives 6 values per round: planning, lock + slot
+ * search, patching the node, hipGraphLaunch, launch-returned-to-completion-seen,
+ * and the whole round.  The counters and the word are allocated here (bench
+ * code; the component's own come from its event pool).
+ */
+typedef xccl_status_t (*graph_flagged_fn_t)(void *, void *, void *, size_t, size_t, size_t, xccl_dt_t, xccl_op_t,
+                                            void *, uint32_t *, uint32_t *, uint32_t, int *, uint64_t *);
+
+xccl_status_t xccl_rocm_bench_graph_parts(xccl_rocm_mem_component_t *mc, graph_flagged_fn_t graph_fn, void *sbuf1,
+                                          void *sbuf2, void *rbuf, size_t count, size_t size, size_t stride,
+                                          xccl_dt_t dtype, xccl_op_t op, size_t iters, uint64_t *ns_out)
+{
+    void              *stream = NULL;
+    uint32_t          *counters = NULL, *dev_flag = NULL;
+    volatile uint32_t *flag = NULL;
+    xccl_status_t      st = mc->get_stream(&stream);
+    size_t             i;
+
+    if (st != XCCL_OK) {
+        return st;
+    }
+    if (hipMalloc((void **)&counters, XCCL_ROCM_DONE_COUNT_BYTES) != hipSuccess ||
+        hipMemset(counters, 0, XCCL_ROCM_DONE_COUNT_BYTES) != hipSuccess ||
+        hipHostMalloc((void **)&flag, 64, hipHostMallocMapped) != hipSuccess ||
+        hipHostGetDevicePointer((void **)&dev_flag, (void *)flag, 0) != hipSuccess) {
+        return XCCL_ERR_NO_MESSAGE;
+    }
+    *flag = 0;
+    for (i = 0; i < iters && st == XCCL_OK; i++) {
+        uint64_t       parts[4] = {0, 0, 0, 0};
+        int            flagged  = 0;
+        const uint64_t t0       = now_ns();
+        uint64_t       t1;
+        st = graph_fn(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, stream, counters, dev_flag, (uint32_t)(i + 1),
+                      &flagged, parts);
+        t1 = now_ns();
+        if (st != XCCL_OK) {
+            break;
+        }
+        if (flagged) {
+            while (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != (uint32_t)(i + 1)) {
+            }
+        } else if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) {
+            st = XCCL_ERR_NO_MESSAGE;
+        }
+        ns_out[6 * i + 0] = parts[0];
+        ns_out[6 * i + 1] = parts[1];
+        ns_out[6 * i + 2] = parts[2];
+        ns_out[6 * i + 3] = parts[3];
+        ns_out[6 * i + 4] = now_ns() - t1;
+        ns_out[6 * i + 5] = now_ns() - t0;
+    }
+    (void)hipStreamSynchronize((hipStream_t)stream);
+    (void)hipFree(counters);
+    (void)hipHostFree((void *)flag);
+    return st;
 }

@@ -80,7 +80,59 @@ __global__ void __launch_bounds__(256) copy_kernel(const uint4 *src, uint4 *dst,
     }
 }
 
+// Reads what a reduction of `nsrc` vectors reads, in the same pattern (one
+// wave per 1 KiB tile, the sources one after the other, non-temporal buffer
+// loads, two in flight), and writes nothing: the read-only ceiling that the
+// reduction's read-mostly mix is compared with.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(64) read_kernel(const char *src, size_t stride, uint32_t nsrc, size_t nvec,
+                                                  uint32_t *sink)
+{
+    const size_t v0 = (size_t)blockIdx.x * 64;
+    if (v0 >= nvec) {
+        return;
+    }
+    const size_t   left  = nvec - v0;
+    const uint32_t bytes = (uint32_t)(left < 64 ? left : 64) * 16u;
+    const uint32_t off   = threadIdx.x * 16u;
+    const char    *p     = src + v0 * 16;
+    u32x4          acc   = {0, 0, 0, 0};
+    u32x4          l0    = __builtin_amdgcn_raw_buffer_load_b128(
+        __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, (int)bytes, 0x00027000), (int)off, 0, 2);
+    for (uint32_t j = 1; j <= nsrc; ++j) {
+        p += stride;
+        u32x4 l1 = __builtin_amdgcn_raw_buffer_load_b128(
+            __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, j < nsrc ? (int)bytes : 0, 0x00027000), (int)off, 0, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        acc ^= l0;
+        l0 = l1;
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5eed1234u && sink != nullptr) {
+        *sink = acc.x; // practically never; keeps the loads alive
+    }
+}
+
 } // namespace
+
+// Reads `nsrc` vectors of `bytes` each (a multiple of 16), `stride` bytes apart, with read_kernel on
+// `hip_stream`; `lds_bytes` of unused LDS per workgroup bound the resident waves like the reduction's launch.
+extern "C" xccl_status_t xccl_rocm_bench_read(const void *src, size_t stride, unsigned nsrc, size_t bytes,
+                                              unsigned lds_bytes, void *sink, void *hip_stream)
+{
+    if (bytes % 16 != 0 || nsrc == 0) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    const size_t nvec = bytes / 16;
+    const size_t grid = (nvec + 63) / 64;
+    if (grid == 0 || grid > 0x7fffffffu) {
+        return XCCL_ERR_INVALID_PARAM;
+    }
+    hipLaunchKernelGGL(read_kernel, dim3((unsigned)grid), dim3(64), lds_bytes, (hipStream_t)hip_stream,
+                       (const char *)src, stride, nsrc, nvec, (uint32_t *)sink);
+    return hipGetLastError() == hipSuccess ? XCCL_OK : XCCL_ERR_NO_MESSAGE;
+}
 
 // Copies `bytes` (a multiple of 16) from src to dst with copy_kernel on `hip_stream`.
 extern "C" xccl_status_t xccl_rocm_bench_copy(void *dst, const void *src, size_t bytes, void *hip_stream)

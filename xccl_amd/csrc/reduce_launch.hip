@@ -19,10 +19,9 @@ constexpr int kMaxDevices       = 64;
 // workgroup measured fastest, so the cap only bounds the grid of huge calls.
 constexpr int kDefaultBlocksPerCu = 8192;
 
-// Resident one-wave workgroups per compute unit for large launches, by source
-// count (0 = these defaults, > 0 = this many for every call, >= kNoResidentCap =
-// no cap).  Measured on MI355X with the source-by-source walk: no cap for 2
-// sources, 16 for 3-4, 24 beyond.
+// Resident one-wave workgroups per compute unit for large launches (0 = the
+// defaults of lds_for_resident, > 0 = this many for every call,
+// >= kNoResidentCap = no cap).
 constexpr int    kNoResidentCap = 32;
 constexpr size_t kLdsPerCu      = 160 * 1024;
 constexpr size_t kLdsPerGroup   = 64 * 1024; // most a workgroup may ask for
@@ -141,11 +140,18 @@ struct Plan {
 };
 
 // LDS per workgroup that lets `resident` workgroups share a compute unit.
-unsigned lds_for_resident(uint32_t nsrc, size_t grid, int cus)
+// `footprint`: bytes the call touches.  Measured (fp32/fp64/fp16 SUM, 256 MiB
+// vectors, rotating destination): 2 sources want every wave slot (7.0 TB/s
+// against 6.4 at 16), 3 sources 20 (6.76), 4 to 16 sources 16 (6.6-6.76; 6.2-6.5
+// without a cap).  A call whose vectors all fit the 256 MB memory-side cache
+// (the integer sweep's 16 Mi-element vectors of 1 and 2 bytes) is served from
+// there when its operands were just written, and wants every slot as well
+// (int8 SUM, 4 sources: 6.86 TB/s against 6.26 at 16).
+unsigned lds_for_resident(uint32_t nsrc, size_t grid, int cus, size_t footprint)
 {
     int cap = g_resident.load(std::memory_order_relaxed);
     if (cap == 0) {
-        cap = nsrc <= 2 ? kNoResidentCap : nsrc <= 4 ? 16 : 24;
+        cap = (nsrc <= 2 || footprint <= ((size_t)192 << 20)) ? kNoResidentCap : nsrc == 3 ? 20 : 16;
     }
     if (cap >= kNoResidentCap || grid <= (size_t)cap * (size_t)cus) {
         return 0; // the whole grid is resident at once anyway
@@ -238,7 +244,7 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
         grid = 1; // head/tail only
     }
     plan->grid      = (unsigned)grid;
-    plan->lds_bytes = lds_for_resident(nsrc, grid, cus);
+    plan->lds_bytes = lds_for_resident(nsrc, grid, cus, (size_t)(nsrc + 1) * elems * esize);
     plan->fn        = e->fn;
     return XCCL_OK;
 }

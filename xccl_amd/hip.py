@@ -67,6 +67,14 @@ def host_malloc(nbytes: int) -> int:
     return p.value
 
 
+def host_get_device_pointer(host_ptr: int) -> int:
+    """Device view of memory from host_malloc."""
+    p = ctypes.c_void_p()
+    check(lib().hipHostGetDevicePointer(ctypes.byref(p), ctypes.c_void_p(host_ptr), ctypes.c_uint(0)),
+          "hipHostGetDevicePointer")
+    return p.value
+
+
 def host_free(ptr: int):
     check(lib().hipHostFree(ctypes.c_void_p(ptr)), "hipHostFree")
 

@@ -156,10 +156,14 @@ def benchkit_lib():
         lib.xccl_rocm_bench_latency.argtypes = [_vp, _vp, _int, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
         lib.xccl_rocm_bench_kernel_times.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp]
         lib.xccl_rocm_bench_region_time.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp, _vp, _vp]
+        lib.xccl_rocm_bench_region_time_rot.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _int, _int, _sz,
+                                                        _vp, _vp, _vp]
         lib.xccl_rocm_bench_latency_mt.argtypes = [_vp, _int, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
         lib.xccl_rocm_bench_memcpy.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _vp]
         lib.xccl_rocm_bench_mem_type.argtypes = [_vp, _vp, _sz, _vp, _vp]
         lib.xccl_rocm_bench_alloc_free.argtypes = [_vp, _sz, _sz, _vp]
+        lib.xccl_rocm_bench_graph_parts.argtypes = [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _sz, _vp]
+        lib.xccl_rocm_bench_read.argtypes = [_vp, _sz, _c.c_uint, _sz, _c.c_uint, _vp, _vp]
         _datagen_lib = lib
     return _datagen_lib
 
@@ -323,6 +327,19 @@ def bench_kernel_times(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters
     return _st(st), out
 
 
+def bench_region_time_rot(sbuf1, sbuf2, rbuf, rot_count, rot_pitch, count, size, stride, dtype, op, iters: int):
+    """bench_region_time with the destination cycling through `rot_count` vectors `rot_pitch` bytes apart."""
+    from . import hip
+    e0, e1 = hip.event_create(), hip.event_create()
+    ms = _c.c_float(0)
+    st = benchkit_lib().xccl_rocm_bench_region_time_rot(_c.addressof(component()), sbuf1, sbuf2, rbuf, rot_count,
+                                                        rot_pitch, count, size, stride, int(dtype), int(op), iters,
+                                                        e0, e1, _c.byref(ms))
+    hip.event_destroy(e0)
+    hip.event_destroy(e1)
+    return _st(st), ms.value
+
+
 def bench_region_time(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters: int):
     """Device time in ms of `iters` back-to-back launches on the component stream,
     from ONE pair of HIP events around them all."""
@@ -334,6 +351,22 @@ def bench_region_time(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters:
     hip.event_destroy(e0)
     hip.event_destroy(e1)
     return _st(st), ms.value
+
+
+def bench_graph_parts(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters: int):
+    """Host time in ns of the steps of a one-node graph launch with a completion word, `iters` rounds x
+    (planning, lock + slot search, patching, hipGraphLaunch, completion seen, whole round)."""
+    import numpy as np
+    out = np.zeros((iters, 6), dtype=np.uint64)
+    fn = _c.cast(component_lib().xccl_rocm_reduce_multi_graph_flagged, _vp)
+    st = benchkit_lib().xccl_rocm_bench_graph_parts(_c.addressof(component()), fn, sbuf1, sbuf2, rbuf, count, size,
+                                                    stride, int(dtype), int(op), iters, out.ctypes.data)
+    return _st(st), out
+
+
+def bench_read(src, stride, nsrc, nbytes, lds_bytes=0, hip_stream=None) -> Status:
+    """Read-only kernel with the reduction's access pattern (nothing is written)."""
+    return _st(benchkit_lib().xccl_rocm_bench_read(src, stride, nsrc, nbytes, lds_bytes, None, hip_stream))
 
 
 def bench_latency_mt(threads: int, thread_pitch: int, sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters: int):
