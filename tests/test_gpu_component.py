@@ -294,6 +294,40 @@ def test_stream_gate_times_out_by_itself(rocm):
     hip.host_free(flag_host)
 
 
+def test_finish_stream_activity_reports_a_gate_that_gave_up():
+    """A gate whose time limit passes before finish_stream_activity let the
+    user's stream run early; finish must say so (XCCL_ERR_NO_PROGRESS) instead
+    of returning XCCL_OK.  The limit comes from the environment, read once per
+    process, hence a child process with a 30 ms limit; the gate kernel leaves
+    by itself, nothing is left spinning."""
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import sys, time\n"
+        "sys.path.insert(0, %r)\n"
+        "from xccl_amd import hip, mc\n"
+        "from xccl_amd.types import Status\n"
+        "hip.set_device(0)\n"
+        "assert mc.xccl_mem_component_init() == Status.OK\n"
+        "s = mc.Stream(hip.stream_create())\n"
+        "st, req = mc.xccl_mem_component_start_acitivity(s)\n"
+        "assert st == Status.OK\n"
+        "hip.stream_synchronize(s.hip_stream)\n"       # returns once the gate has given up
+        "late = mc.xccl_mem_component_finish_acitivity(req)\n"
+        "st, req = mc.xccl_mem_component_start_acitivity(s)\n"
+        "assert st == Status.OK\n"
+        "in_time = mc.xccl_mem_component_finish_acitivity(req)\n"
+        "hip.stream_synchronize(s.hip_stream)\n"
+        "print('late', int(late), 'in_time', int(in_time))\n"
+    ) % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, XCCL_MC_ROCM_GATE_TIMEOUT_MS="30")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "late %d in_time %d" % (int(Status.ERR_NO_PROGRESS), int(Status.OK)) in out.stdout, out.stdout + out.stderr
+    assert "stream gate gave up" in out.stderr
+
+
 @pytest.mark.parametrize("dt", [Dt.INT8, Dt.UINT16, Dt.INT32, Dt.UINT64, Dt.FLOAT16, Dt.FLOAT32, Dt.FLOAT64],
                          ids=lambda d: Dt(d).name)
 def test_datagen_matches_oracle_generator(rocm, oracle, dt):

@@ -166,3 +166,53 @@ def test_vectors_beyond_4GiB(rocm, oracle):
             assert np.array_equal(dev.download(np.uint8, 8192, 2 * stride + lo), a ^ b)
     finally:
         dev.close()
+
+
+def test_config5_small_message_grid(rocm, oracle):
+    """The small-message sweep as a parity test: FLOAT32 SUM, 2, 4 and 8
+    sources, 4 B .. 32 KiB per vector in powers of two, through the three ways
+    a call can complete -- the blocking entry, reduce_multi_nb + event polling,
+    and the single-node graph launch -- each bit-exact against the oracle's
+    same-order fold."""
+    maxb = 32768
+    lib = rocm.component_lib()
+    stream = rocm.component_stream()
+    slab = oracle.slab(8, maxb // 4, Dt.FLOAT32, 5)
+    dev = hip.DeviceBuffer(9 * maxb)
+    dev.upload(slab)
+    dst = dev.ptr + 8 * maxb
+    want = np.empty(maxb // 4, dtype=np.float32)
+    try:
+        for nsrc in (2, 4, 8):
+            for k in range(14):
+                nbytes = 4 << k
+                cnt = nbytes // 4
+                oracle.reduce_multi(slab, slab, want, nsrc - 1, cnt, maxb, Dt.FLOAT32, Op.SUM, off2=maxb)
+                for mode in ("sync", "event", "graph"):
+                    hip.memset(dst, 0xEE, maxb)
+                    hip.device_synchronize()
+                    if mode == "sync":
+                        st = rocm.xccl_mem_component_reduce_multi(dev.ptr, dev.ptr + maxb, dst, nsrc - 1, cnt, maxb,
+                                                                  Dt.FLOAT32, Op.SUM, MemType.ROCM)
+                        assert st == Status.OK
+                    elif mode == "event":
+                        st, ev = rocm.xccl_mem_component_reduce_multi_nb(dev.ptr, dev.ptr + maxb, dst, nsrc - 1, cnt, maxb,
+                                                                         Dt.FLOAT32, Op.SUM, MemType.ROCM)
+                        assert st == Status.OK and ev
+                        while True:
+                            q = rocm.xccl_mc_event_query(ev)
+                            if q != Status.INPROGRESS:
+                                break
+                        assert q == Status.OK
+                        assert rocm.xccl_mc_event_free(ev) == Status.OK
+                    else:
+                        st = lib.xccl_rocm_reduce_multi_graph(dev.ptr, dev.ptr + maxb, dst, nsrc - 1, cnt, maxb,
+                                                              int(Dt.FLOAT32), int(Op.SUM), stream)
+                        assert st == Status.OK
+                        hip.stream_synchronize(stream)
+                    got = dev.download(np.float32, maxb // 4, 8 * maxb)
+                    assert got[:cnt].tobytes() == want[:cnt].tobytes(), (nsrc, nbytes, mode)
+                    assert (got[cnt:].view(np.uint8) == 0xEE).all(), "bytes behind the result written: %s" % ((nsrc, nbytes, mode),)
+    finally:
+        dev.close()
+        lib.xccl_rocm_graph_cache_destroy()

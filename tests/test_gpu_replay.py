@@ -8,7 +8,7 @@ import pytest
 
 from gpu_util import NP
 from xccl_amd import hip
-from xccl_amd.types import Dt, Op, Status, dt_size
+from xccl_amd.types import Dt, Op, Status, dt_size, supported_pairs, FP_DTYPES
 
 pytestmark = pytest.mark.gpu
 
@@ -117,6 +117,76 @@ def test_order_independent_operators_and_ragged_sizes(rocm, oracle, alg):
             who = range(P) if alg in ALLREDUCE else [P // 2]
             for r in who:
                 assert rk.result(r).tobytes() == want.tobytes(), (alg, P, radix, count, Dt(dt).name, Op(op).name, r)
+            rk.close()
+
+
+def _expected_any_order(host, dt, op):
+    """The reduction over the rank axis for an operator whose bits do not
+    depend on the fold order, computed by numpy alone; for floating-point SUM
+    and PROD (order-dependent) a float64 value and an error bound instead."""
+    P = host.shape[0]
+    if int(dt) in [int(d) for d in FP_DTYPES] and op in (Op.SUM, Op.PROD):
+        x = host.astype(np.float64)
+        u = {2: 2.0 ** -11, 4: 2.0 ** -24, 8: 2.0 ** -53}[host.itemsize]
+        tiny = float(np.finfo(host.dtype).smallest_subnormal)
+        # binary64 inputs: the float64 value below carries P-1 roundings of its own, hence twice the bound
+        k = (2 if host.itemsize == 8 else 1) * (P - 1)
+        if op == Op.SUM:
+            return x.sum(axis=0), k * u * np.abs(x).sum(axis=0) + k * tiny
+        # every multiplication is off by at most u relative (to first order), or half a subnormal step absolute
+        return x.prod(axis=0), 1.01 * k * u * np.abs(x.prod(axis=0)) + k * tiny
+    with np.errstate(over="ignore"):
+        if op == Op.SUM:
+            return np.add.reduce(host, axis=0, dtype=host.dtype), None
+        if op == Op.PROD:
+            return np.multiply.reduce(host, axis=0, dtype=host.dtype), None
+    if op == Op.MAX:
+        return np.maximum.reduce(host, axis=0), None
+    if op == Op.MIN:
+        return np.minimum.reduce(host, axis=0), None
+    if op == Op.BAND:
+        return np.bitwise_and.reduce(host, axis=0), None
+    if op == Op.BOR:
+        return np.bitwise_or.reduce(host, axis=0), None
+    if op == Op.BXOR:
+        return np.bitwise_xor.reduce(host, axis=0), None
+    truth = host != 0
+    if op == Op.LAND:
+        return truth.all(axis=0).astype(host.dtype), None
+    if op == Op.LOR:
+        return truth.any(axis=0).astype(host.dtype), None
+    assert op == Op.LXOR
+    return (truth.sum(axis=0) % 2).astype(host.dtype), None
+
+
+@pytest.mark.parametrize("stream_ordered", [False, True], ids=["blocking", "stream_ordered"])
+@pytest.mark.parametrize("alg", ALLREDUCE + REDUCE)
+def test_every_dtype_op_through_every_call_site(rocm, oracle, alg, stream_ordered):
+    """test_mpi_cuda_allreduce.c:45-76 / test_mpi_cuda_reduce.c:47-78 "for every
+    (dtype, op)": all 92 supported pairs through each algorithm's call sites
+    (their in-place aliasing and scratch strides included), 5 ranks at radix 4
+    (one extra rank handing its vector to a proxy) and 8 ranks at radix 4, a
+    count that leaves ragged segments.  Integer operators, and floating-point
+    MAX/MIN, must match numpy's reduction bit for bit whatever tree the
+    algorithm builds; floating-point SUM/PROD must lie within the error bound
+    of P-1 roundings."""
+    count = 257
+    for P in (5, 8):
+        root = P - 2
+        for dt, op in supported_pairs():
+            sparse = op in (Op.LAND, Op.LOR, Op.LXOR)
+            host = np.stack([oracle.fill(count, dt, 900 + P, r, sparse) for r in range(P)])
+            want, bound = _expected_any_order(host, dt, op)
+            rk = Ranks(host)
+            st, _ = rocm.replay_run(alg, rk.src_ptrs(), rk.dst_ptrs(), count, dt, op, radix=4, root=root,
+                                    stream_ordered=stream_ordered)
+            assert st == Status.OK, (alg, P, Dt(dt).name, Op(op).name, st)
+            for r in (range(P) if alg in ALLREDUCE else [root]):
+                got = rk.result(r)
+                if bound is None:
+                    assert got.tobytes() == want.tobytes(), (alg, P, Dt(dt).name, Op(op).name, r)
+                else:
+                    assert (np.abs(got.astype(np.float64) - want) <= bound).all(), (alg, P, Dt(dt).name, Op(op).name, r)
             rk.close()
 
 
@@ -261,3 +331,12 @@ def test_c_program_in_the_shape_of_the_reference_tests():
         out = subprocess.run([exe, LIB_DIR, str(team), str(count)], capture_output=True, text=True, timeout=120)
         assert out.returncode == 0, out.stdout + out.stderr
         assert "Correctness check: PASSED" in out.stdout
+    # "... then every (dtype, op)": 8 integer types x 10 operators + FLOAT32/FLOAT64 x MAX, MIN, SUM = 86 cases,
+    # each through the four algorithms in both reduction modes
+    for team, count in ((8, 32), (5, 1001)):
+        out = subprocess.run([exe, LIB_DIR, str(team), str(count), "ALL", "ALL"], capture_output=True, text=True,
+                             timeout=300)
+        assert out.returncode == 0, out.stdout + out.stderr
+        assert "Correctness check: PASSED" in out.stdout and "86 dtype/op cases" in out.stdout
+    out = subprocess.run([exe, LIB_DIR, "4", "64", "UINT16", "LXOR"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and "1 dtype/op case)" in out.stdout, out.stdout + out.stderr
