@@ -65,7 +65,7 @@ xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf,
  * launch writes the word itself: its workgroups count their arrivals in
  * `dev_count`, XCCL_ROCM_DONE_COUNT_BYTES of zeroed device memory (two
  * levels, one counter per 128-byte line), which the kernel leaves zero again.
- * Behind a larger launch (more than 1024 workgroups; XCCL_MC_ROCM_MAX_COUNTED_GRID)
+ * Behind a larger launch (more than 2048 workgroups; XCCL_MC_ROCM_MAX_COUNTED_GRID)
  * a one-lane kernel is queued that stores the word, provided every result
  * store of that launch is a write-through vector store (no peeled head or
  * tail elements: 16-byte-aligned operands and a byte count that is a multiple
