@@ -117,8 +117,8 @@ xccl_status_t xccl_rocm_reduce_multi_graph(void *sbuf1, void *sbuf2, void *rbuf,
 /* The graph launch with the completion word of xccl_rocm_reduce_multi_flagged
  * (launches of up to 8192 workgroups; `*flagged` tells) and, for measurement,
  * the host time of its steps in `ns_parts` (may be NULL; 4 values:
- * planning, lock + slot search, building or patching the graph,
- * hipGraphLaunch).  The sequence number is a kernel argument, so a flagged
+ * planning, lock + slot search, building or patching the graph -- which
+ * first waits for the slot's previous launch --, hipGraphLaunch).  The sequence number is a kernel argument, so a flagged
  * launch patches its node on every call. */
 xccl_status_t xccl_rocm_reduce_multi_graph_flagged(void *sbuf1, void *sbuf2, void *rbuf,
                                                    size_t count, size_t size,

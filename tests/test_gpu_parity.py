@@ -22,9 +22,10 @@ def _id(p):
 
 @pytest.mark.parametrize("pair", ALL_PAIRS, ids=_id)
 def test_every_dtype_op_small(rocm, oracle, pair):
-    """Every supported (dtype, op): source counts on and off the specialised
-    kernels (2, 3, 4, 8, 16 sources vs 5, 9, 17), sizes around the 16-byte
-    vector and the 128-vector tile of a one-wave workgroup."""
+    """Every supported (dtype, op): even and odd source counts (the walk
+    through the sources alternates between two load registers), 2 to 17
+    sources, sizes around the 16-byte vector and the 64-vector tile of a
+    one-wave workgroup."""
     dt, op = pair
     for n2, size in ((1, 1), (1, 1000), (2, 37), (3, 4099), (4, 513), (7, 2048 + 5), (8, 700), (15, 1031),
                      (16, 129)):

@@ -404,9 +404,9 @@ xccl_status_t graph_launch(Plan &plan, hipStream_t stream, uint64_t *ns)
             }
             victim->live = true;
         } else {
-            // The executable graph may still be running its previous launch
-            // on another stream; patch it only once that launch has finished.
-            if (victim->last_stream_valid && victim->last_stream != stream) {
+            // The executable graph may still be running its previous launch;
+            // patch it only once that launch has finished.
+            if (victim->last_stream_valid) {
                 HIP_OR_FAIL(hipStreamSynchronize(victim->last_stream));
             }
             victim->plan = plan;
