@@ -117,6 +117,33 @@ template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBand>(u32x4 a, u32
 template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBor>(u32x4 a, u32x4 b)  { return a | b; }
 template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpBxor>(u32x4 a, u32x4 b) { return a ^ b; }
 
+// 8- and 16-bit elements, four or two to a register: the logical operators and
+// the 8-bit SUM as whole-register arithmetic.  Element by element the compiler
+// unpacks and repacks every byte (about 40 VALU instructions per 16-byte vector
+// and source for LAND), which made these the slowest rows of the integer sweep.
+//   nz(x): 1 in every element of x that is non-zero, else 0 -- adding 0x7f..
+//   to the low bits carries into an element's top bit iff they are non-zero.
+__device__ __forceinline__ u32x4 nz8(u32x4 x)
+{
+    return ((((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) >> 7) & 0x01010101u;
+}
+__device__ __forceinline__ u32x4 nz16(u32x4 x)
+{
+    return ((((x & 0x7fff7fffu) + 0x7fff7fffu) | x) >> 15) & 0x00010001u;
+}
+template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpLand>(u32x4 a, u32x4 b) { return nz8(a) & nz8(b); }
+template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpLor>(u32x4 a, u32x4 b)  { return nz8(a | b); }
+template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpLxor>(u32x4 a, u32x4 b) { return nz8(a) ^ nz8(b); }
+template <> __device__ __forceinline__ u32x4 vfold<uint16_t, OpLand>(u32x4 a, u32x4 b) { return nz16(a) & nz16(b); }
+template <> __device__ __forceinline__ u32x4 vfold<uint16_t, OpLor>(u32x4 a, u32x4 b)  { return nz16(a | b); }
+template <> __device__ __forceinline__ u32x4 vfold<uint16_t, OpLxor>(u32x4 a, u32x4 b) { return nz16(a) ^ nz16(b); }
+// byte-wise wrapping add: add the low 7 bits of every byte (no carry can leave
+// a byte), then put the top bits back with an exclusive or
+template <> __device__ __forceinline__ u32x4 vfold<uint8_t, OpSum>(u32x4 a, u32x4 b)
+{
+    return ((a & 0x7f7f7f7fu) + (b & 0x7f7f7f7fu)) ^ ((a ^ b) & 0x80808080u);
+}
+
 // Vector accesses go through buffer instructions: the descriptor (scalar
 // registers) holds the tile's base address and its length in bytes, the lane
 // supplies a 32-bit offset.  The hardware drops stores and returns zero for
