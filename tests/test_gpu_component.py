@@ -543,3 +543,46 @@ def test_stream_ordered_entries_under_stream_capture(rocm, oracle):
     finally:
         c.close()
         hip.stream_destroy(s.hip_stream)
+
+
+def test_first_use_of_a_device_inside_a_capture_is_refused():
+    """The component creates its per-device stream, events and counters on the
+    first call on a device, which allocates and synchronises; inside a stream
+    capture that would invalidate the capture.  A fresh process whose first
+    call arrives with a capturing stream gets XCCL_ERR_NO_RESOURCE and an
+    intact capture; after one call outside a capture the same capture works."""
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import sys\n"
+        "sys.path.insert(0, %r)\n"
+        "import numpy as np\n"
+        "from xccl_amd import hip, mc\n"
+        "from xccl_amd.types import Dt, MemType, Op, Status\n"
+        "hip.set_device(0)\n"
+        "assert mc.xccl_mem_component_init() == Status.OK\n"
+        "buf = hip.DeviceBuffer(3 * 4096)\n"
+        "buf.upload(np.arange(2048, dtype=np.float32))\n"
+        "s = mc.Stream(hip.stream_create())\n"
+        "args = (buf.ptr, buf.ptr + 4096, buf.ptr + 8192, 1, 1024, 4096, Dt.FLOAT32, Op.SUM, MemType.ROCM, s)\n"
+        "hip.stream_begin_capture(s.hip_stream)\n"
+        "first, _ = mc.xccl_mem_component_reduce_multi_nb(*args, want_event=False)\n"
+        "g = hip.stream_end_capture(s.hip_stream)\n"          # the capture itself must have survived
+        "hip.graph_destroy(g)\n"
+        "warm = mc.xccl_mem_component_reduce_multi(*args[:9])\n"
+        "hip.stream_begin_capture(s.hip_stream)\n"
+        "second, _ = mc.xccl_mem_component_reduce_multi_nb(*args, want_event=False)\n"
+        "g = hip.stream_end_capture(s.hip_stream)\n"
+        "ge = hip.graph_instantiate(g)\n"
+        "hip.memset(buf.ptr + 8192, 0, 4096)\n"
+        "hip.graph_launch(ge, s.hip_stream)\n"
+        "hip.stream_synchronize(s.hip_stream)\n"
+        "got = buf.download(np.float32, 1024, 8192)\n"
+        "ok = bool((got == np.arange(1024, dtype=np.float32) + np.arange(1024, 2048, dtype=np.float32)).all())\n"
+        "print('first', int(first), 'warm', int(warm), 'second', int(second), 'replay', ok)\n"
+    ) % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "first %d warm 0 second 0 replay True" % int(Status.ERR_NO_RESOURCE) in out.stdout, out.stdout + out.stderr
+    assert "inside a stream capture" in out.stderr

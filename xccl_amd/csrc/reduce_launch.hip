@@ -165,7 +165,8 @@ bool same_plan(const Plan &a, const Plan &b)
     return a.fn == b.fn && a.grid == b.grid && a.lds_bytes == b.lds_bytes && a.args.s1 == b.args.s1 && a.args.s2 == b.args.s2 &&
            a.args.dst == b.args.dst && a.args.stride == b.args.stride && a.args.head == b.args.head &&
            a.args.nvec == b.args.nvec && a.args.tail == b.args.tail && a.args.n2 == b.args.n2 &&
-           a.args.done_flag == b.args.done_flag && a.args.done_seq == b.args.done_seq;
+           a.args.done_flag == b.args.done_flag && a.args.done_count == b.args.done_count &&
+           a.args.done_seq == b.args.done_seq;
 }
 
 // Bytes to peel so that as many of the buffers as possible start their
