@@ -586,3 +586,57 @@ def test_first_use_of_a_device_inside_a_capture_is_refused():
     assert out.returncode == 0, out.stdout + out.stderr
     assert "first %d warm 0 second 0 replay True" % int(Status.ERR_NO_RESOURCE) in out.stdout, out.stdout + out.stderr
     assert "inside a stream capture" in out.stderr
+
+
+def test_graph_launch_with_completion_word(rocm, oracle):
+    """xccl_rocm_reduce_multi_graph_flagged: the one-node graph launch that
+    carries the kernel-written completion word (its sequence number is a kernel
+    argument, so every call patches the node) and reports the host time of its
+    steps.  Same bits as the oracle on every call, the word written last."""
+    lib = rocm.component_lib()
+    stream = rocm.component_stream()
+    host_word = hip.host_malloc(64)
+    ctypes.memset(host_word, 0, 64)
+    dev_word = hip.host_get_device_pointer(host_word)
+    counters = hip.malloc((1 + 64) * 128)
+    hip.memset(counters, 0, (1 + 64) * 128)
+    hip.device_synchronize()
+    word = ctypes.cast(host_word, ctypes.POINTER(ctypes.c_uint32))
+    cases = []
+    try:
+        seq = 0
+        for k, (dt, op, size, n2) in enumerate(((Dt.FLOAT32, Op.SUM, 4099, 3), (Dt.INT16, Op.MIN, 100000, 7),
+                                                (Dt.FLOAT32, Op.SUM, 4099, 3), (Dt.UINT8, Op.LAND, 77, 1))):
+            c = Case(dt, size, n2)
+            c.fill_random(oracle, 90 + k, op)
+            c.upload()
+            cases.append(c)
+            p1, p2, pr = c.ptrs()
+            want, _ = c.expect(oracle, op)
+            for rep in range(2):
+                hip.memset(pr, 0xEE, c.vbytes)
+                hip.device_synchronize()
+                seq += 1
+                flagged = ctypes.c_int(0)
+                parts = (ctypes.c_uint64 * 4)()
+                st = lib.xccl_rocm_reduce_multi_graph_flagged(p1, p2, pr, n2, size, c.stride, int(dt), int(op), stream,
+                                                              counters, dev_word, seq, ctypes.byref(flagged), parts)
+                assert st == Status.OK and flagged.value == 1
+                t0 = time.time()
+                while word[0] != seq:
+                    assert time.time() - t0 < 20.0, "completion word never written"
+                assert_same(c.result(), want, dt, op, "graph + completion word, %s %s rep %d" % (dt.name, op.name, rep))
+                assert parts[3] > 0        # hipGraphLaunch took measurable host time
+        # without a word it is the plain graph launch
+        c = cases[0]
+        p1, p2, pr = c.ptrs()
+        assert lib.xccl_rocm_reduce_multi_graph_flagged(p1, p2, pr, c.n2, c.size, c.stride, int(Dt.FLOAT32), int(Op.SUM),
+                                                        stream, None, None, 0, None, None) == Status.OK
+        hip.stream_synchronize(stream)
+    finally:
+        hip.stream_synchronize(stream)
+        for c in cases:
+            c.close()
+        lib.xccl_rocm_graph_cache_destroy()
+        hip.free(counters)
+        hip.host_free(host_word)
