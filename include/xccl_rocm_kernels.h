@@ -37,6 +37,14 @@
 extern "C" {
 #endif
 
+/* Looks up what the launchers need to know about the CURRENT device (its
+ * compute-unit count, the address of the library's static counter array on
+ * it) so that later calls on that device make no runtime query.  Optional:
+ * the launchers do the same on their first call on a device; a caller that
+ * will launch from inside a stream capture calls this once outside it.  The
+ * component calls it when it sets a device up. */
+xccl_status_t xccl_rocm_prepare_device(void);
+
 /* XCCL_OK if a kernel exists for (dtype, op), XCCL_ERR_UNSUPPORTED if not.
  * Host-only; touches no device.  Same matrix as the two launchers below. */
 xccl_status_t xccl_rocm_reduce_supported(xccl_dt_t dtype, xccl_op_t op);
@@ -96,6 +104,8 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
  * one is through.  Limit: at most 8192 workgroups, i.e. 8 MiB per vector; a
  * larger call returns XCCL_ERR_INVALID_PARAM and prints why.  Every call on a
  * GPU shares that GPU's array: calls that overlap in time on one GPU race.
+ * The array's address on a device is looked up on the first call there (or by
+ * xccl_rocm_prepare_device): make that one outside any capture.
  */
 xccl_status_t xccl_rocm_reduce_multi_flagged_static(void *sbuf1, void *sbuf2, void *rbuf,
                                                     size_t count, size_t size,

@@ -222,6 +222,11 @@ static xccl_status_t mc_rocm_device_create_parts(mc_rocm_device_t *d)
 {
     int i;
 
+    xccl_status_t st = xccl_rocm_prepare_device(); /* compute-unit count, static counter array */
+
+    if (st != XCCL_OK) {
+        return st;
+    }
     MC_HIP(hipStreamCreateWithFlags(&d->stream[0], hipStreamNonBlocking));
     MC_HIP(hipHostMalloc((void **)&d->gate_words,
                          XCCL_ROCM_MC_NUM_STREAM_REQUESTS * sizeof(int),

@@ -517,6 +517,14 @@ __global__ void clear_words_kernel(uint32_t *p, uint32_t n)
 
 extern "C" {
 
+xccl_status_t xccl_rocm_prepare_device(void)
+{
+    int           cus = 0;
+    uint32_t     *p   = nullptr;
+    xccl_status_t st  = cu_count(&cus);
+    return st != XCCL_OK ? st : static_scratch(&p);
+}
+
 xccl_status_t xccl_rocm_reduce_supported(xccl_dt_t dtype, xccl_op_t op)
 {
     return lookup(dtype, op) ? XCCL_OK : XCCL_ERR_UNSUPPORTED;
