@@ -577,7 +577,9 @@ def main():
                      "kernel_ms_avg_event_pair_each": round(float(np.mean(kms)), 4),
                      "achieved_rotating_dst": round(rot, 2), "frac_rotating_dst": round(rot / HBM_PEAK_GBPS, 4),
                      "kernel_ms_avg_rotating_dst": round(rot_us / 1e3, 4),
-                     "frac_of_measured_read_only": round(achieved / peak["read_only_GBps"], 4) if peak else None},
+                     "frac_of_measured_read_only": round(achieved / max(peak["read_only_GBps"],
+                                                                        peak["read_only_no_residency_cap_GBps"]), 4)
+                     if peak else None},
         "measured_peak": peak or None,
     }
 
