@@ -120,7 +120,8 @@ extern "C" {
  * this one launch, not to later replays).  The component creates its
  * per-device resources on the first call on a device, which allocates and
  * synchronises: make that call outside any capture (a call with a capturing
- * `stream` on a device not yet used returns XCCL_ERR_NO_RESOURCE).
+ * `stream` on a device not yet used returns XCCL_ERR_NO_RESOURCE, from these
+ * entries as from event_record and start_stream_activity).
  *
  * finish_stream_activity returns XCCL_ERR_NO_PROGRESS when the gate kernel
  * had already given up (XCCL_MC_ROCM_GATE_TIMEOUT_MS, default 30 s; the

@@ -645,7 +645,7 @@ static xccl_status_t mc_rocm_event_record(xccl_stream_t *stream,
     if (st != XCCL_OK) {
         return st;
     }
-    st = mc_rocm_device(&d);
+    st = mc_rocm_device_for_stream(&d, hs);
     if (st != XCCL_OK) {
         return st;
     }
@@ -735,7 +735,7 @@ mc_rocm_start_stream_activity(xccl_stream_t *stream,
     if (st != XCCL_OK) {
         return st;
     }
-    st = mc_rocm_device(&d);
+    st = mc_rocm_device_for_stream(&d, user);
     if (st != XCCL_OK) {
         return st;
     }
