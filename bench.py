@@ -433,10 +433,7 @@ def profile_mode(a, mc, hip):
 
 
 def plan_of(mc, buf, nsrc, size, stride, dt, op):
-    grid, block, name = mc._c.c_uint(0), mc._c.c_uint(0), mc._c.create_string_buffer(256)
-    mc.component_lib().xccl_rocm_reduce_multi_plan(buf, buf + stride, buf + nsrc * stride, nsrc - 1, size, stride,
-                                                   int(dt), int(op), mc._c.byref(grid), mc._c.byref(block), name, 256)
-    return {"kernel": name.value.decode(), "grid": grid.value, "block": block.value}
+    return mc.reduce_multi_plan(buf, buf + stride, buf + nsrc * stride, nsrc - 1, size, stride, dt, op)
 
 
 def traffic_for(plan):

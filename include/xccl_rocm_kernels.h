@@ -74,14 +74,13 @@ xccl_status_t xccl_rocm_reduce_multi_impl(void *sbuf1, void *sbuf2, void *rbuf,
  * `dev_count`, XCCL_ROCM_DONE_COUNT_BYTES of zeroed device memory (two
  * levels, one counter per 128-byte line), which the kernel leaves zero again.
  * Behind a larger launch (more than 2048 workgroups; XCCL_MC_ROCM_MAX_COUNTED_GRID)
- * a one-lane kernel is queued that stores the word, provided every result
- * store of that launch is a write-through vector store (no peeled head or
- * tail elements: 16-byte-aligned operands and a byte count that is a multiple
- * of 16); launches that are not keep counting up to
- * 8192 workgroups.  Beyond that, or with XCCL_MC_ROCM_TAIL_FLAG=0 in the
- * environment where the queued kernel would be used, or if its launch
- * fails, `*flagged` is 0 and the caller waits for the stream as usual.  One launch at a time per (count, flag) pair.  No
- * counterpart in the reference.
+ * a one-lane kernel is queued that stores the word: every result store of
+ * the reduction is a system-scope write-through store, so the results are in
+ * memory when that kernel starts.  With XCCL_MC_ROCM_TAIL_FLAG=0 in the
+ * environment launches count their arrivals up to 8192 workgroups instead;
+ * beyond that, or if the queued kernel's launch fails, `*flagged` is 0 and
+ * the caller waits for the stream as usual.  One launch at a time per
+ * (count, flag) pair.  No counterpart in the reference.
  */
 #define XCCL_ROCM_DONE_COUNT_BYTES ((1 + 64) * 128)
 xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbuf,
@@ -154,6 +153,15 @@ void xccl_rocm_graph_cache_destroy(void);
  * XCCL_MC_ROCM_RESIDENT_PER_CU), read once at first launch.
  */
 void xccl_rocm_set_launch_shape(int blocks_per_cu, int resident_per_cu);
+
+/*
+ * Launches of at most `max_grid` workgroups with four or more sources run the
+ * burst kernel (every load of a tile issued at once: such a launch is bound by
+ * latency, not by bandwidth); larger ones walk their sources two loads at a
+ * time.  Same results either way.  0 = never, negative = the built-in default;
+ * also XCCL_MC_ROCM_BURST_MAX_GRID.  For measurement and tests.
+ */
+void xccl_rocm_set_burst_max_grid(int max_grid);
 
 /* What a launch with these arguments would be: grid/block size and the
  * mangled kernel name (truncated into `name`, if not NULL).  Host-only apart

@@ -219,6 +219,30 @@ def test_grid_cap_and_ragged_tiles(rocm, oracle):
         lib.xccl_rocm_set_launch_shape(0, 0)
 
 
+def test_walk_and_burst_kernels_agree_with_the_oracle(rocm, oracle):
+    """Small launches with four or more sources run the burst kernel (every
+    load of a tile at once), larger ones the source-by-source walk.  Both are
+    forced onto the same calls -- every supported (dtype, op), source counts
+    around the burst length of 8 and its multiples, ragged sizes, in place --
+    and must give the oracle's bytes."""
+    lib = rocm.component_lib()
+    pairs = supported_pairs()
+    try:
+        for max_grid in (0, 1 << 30):        # never / always (from four sources on)
+            lib.xccl_rocm_set_burst_max_grid(max_grid)
+            for i, (dt, op) in enumerate(pairs):
+                n2 = (3, 7, 8, 9, 15, 16, 17, 24, 25)[i % 9]
+                run_and_check(rocm, oracle, dt, op, 1000 + 37 * i, n2, seed=300 + i,
+                              alias=[None, "s1", ("s2", 0)][i % 3])
+            for n2 in (3, 4, 7, 8, 9, 16, 17, 33):
+                run_and_check(rocm, oracle, Dt.FLOAT32, Op.SUM, 70001, n2, seed=77 + n2, off1=4, offr=8)
+                run_and_check(rocm, oracle, Dt.FLOAT64, Op.MIN, 513, n2, seed=78 + n2)
+            kernel = rocm.reduce_multi_plan(1 << 12, 1 << 13, 1 << 14, 7, 256, 1024, Dt.FLOAT32, Op.SUM)["kernel"]
+            assert kernel.endswith("Lb1EEEvNS_10ReduceArgsE" if max_grid else "Lb0EEEvNS_10ReduceArgsE"), kernel
+    finally:
+        lib.xccl_rocm_set_burst_max_grid(-1)
+
+
 def test_randomised_shapes(rocm, oracle):
     """400 reproducible random calls: any supported (dtype, op), 1..20 vectors
     in sbuf2, sizes up to a few tiles, independent byte placement of the three

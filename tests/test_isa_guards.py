@@ -40,9 +40,18 @@ def _kernels(text):
 
 
 def test_every_variant_is_instantiated(asm):
-    # one kernel per (type, op) family; it takes any number of sources
+    # two kernels per (type, op) family -- the walk and the burst for small launches -- each for any number of sources
     counts = {u: len(_kernels(t)) for u, t in asm.items()}
-    assert counts == {"reduce_w8": 12, "reduce_w16": 9, "reduce_w32": 9, "reduce_w64": 9, "reduce_fp": 12}
+    assert counts == {"reduce_w8": 24, "reduce_w16": 18, "reduce_w32": 18, "reduce_w64": 18, "reduce_fp": 24}
+    for t in asm.values():
+        names = list(_kernels(t))
+        assert sum(_is_burst(n) for n in names) * 2 == len(names)
+
+
+def _is_burst(name):
+    """reduce_multi_kernel<T, Op, true>: the last template argument is mangled as Lb1E."""
+    assert "Lb0EEEv" in name or "Lb1EEEv" in name, name
+    return "Lb1EEEv" in name
 
 
 def _instructions(body):
@@ -60,13 +69,17 @@ def test_completion_word_waits_for_the_result_stores(asm):
             blocks = re.findall(r";;#ASMSTART\n(.*?);;#ASMEND", body, flags=re.S)
             assert [b.strip() for b in blocks] == ["s_waitcnt vmcnt(0)"], (name, blocks)
             wait = body.index(";;#ASMSTART")
-            stores = [m.start() for m in re.finditer(r"\bbuffer_store_dwordx4\b", body)]
+            stores = [m.start() for m in re.finditer(r"\bbuffer_store_\w+\b", body)]
             atomics = [m.start() for m in re.finditer(r"\bglobal_atomic_inc\b", body)]
             publish = [m.start() for m in re.finditer(r"\bglobal_store_dword\b[^\n]* sc0 sc1", body)]
             assert stores and len(atomics) == 2 and len(publish) == 1, (name, len(stores), len(atomics), len(publish))
             assert max(stores) < wait < min(atomics + publish), name
             # nothing branches from the tile loop to behind the wait: the label the loop exits to precedes it
-            assert not re.search(r"\bbuffer_(load|store)_dwordx4\b", body[wait:]), name
+            assert not re.search(r"\bbuffer_(load|store)_\w+\b", body[wait:]), name
+            # every result store is a buffer store with write-through policy: the publishing store (a system-scope
+            # release, which brings the kernel's only cache write-back) is the only global/flat store
+            assert len(re.findall(r"\b(global|flat)_store_\w+", body)) == 1, name
+            assert body.count("buffer_wbl2") == 1, name
 
 
 def test_code_generation_properties(asm):
@@ -79,11 +92,13 @@ def test_code_generation_properties(asm):
             # the tile path moves 16 bytes per lane per access through buffer instructions whose
             # cache-policy bits the compiler sees: non-temporal loads, system-scope write-through stores
             ins = _instructions(body)
-            loads = [i for i in ins if i.startswith("buffer_load_dwordx4")]
-            stores = [i for i in ins if i.startswith("buffer_store_dwordx4")]
-            assert loads and all(i.endswith(" nt") for i in loads), name
-            assert stores and all(i.endswith(" sc0 sc1") for i in stores), name
-            assert "global_load_dwordx4" not in body and "global_store_dwordx4" not in body, name
+            loads = [i for i in ins if i.startswith("buffer_load_")]
+            stores = [i for i in ins if i.startswith("buffer_store_")]
+            assert any(i.startswith("buffer_load_dwordx4") for i in loads) and all(i.endswith(" nt") for i in loads), name
+            assert any(i.startswith("buffer_store_dwordx4") for i in stores) and \
+                all(i.endswith(" sc0 sc1") for i in stores), name
+            # head and tail elements take the same route: no global/flat loads of operands at all
+            assert not re.search(r"\b(global|flat)_load_(u?byte|u?short|dword)", body), name
             # few registers: 24 or more waves fit a compute unit
             assert int(re.search(r"\.amdhsa_next_free_vgpr (\d+)", body).group(1)) <= 80, name
 
@@ -95,6 +110,8 @@ def test_sources_are_walked_with_two_loads_in_flight(asm):
     waits with one load still in flight (vmcnt(1)), not for all of them."""
     for u, text in asm.items():
         for name, body in _kernels(text).items():
+            if _is_burst(name):
+                continue
             run = longest = 0
             for i in _instructions(body):
                 if i.startswith("buffer_load_dwordx4"):
@@ -104,6 +121,23 @@ def test_sources_are_walked_with_two_loads_in_flight(asm):
                     run = 0
             assert longest <= 3, (name, longest)
             assert "s_waitcnt vmcnt(1)" in body, name
+
+
+def test_burst_kernels_issue_every_load_of_a_tile_at_once(asm):
+    """The kernels for small launches ask for sbuf1 and eight vectors of sbuf2
+    before they wait for any of them, and then fold them as they arrive."""
+    for u, text in asm.items():
+        for name, body in _kernels(text).items():
+            if not _is_burst(name):
+                continue
+            run = longest = 0
+            for i in _instructions(body):
+                if i.startswith("buffer_load_dwordx4"):
+                    run += 1
+                    longest = max(longest, run)
+                elif i.startswith("s_waitcnt") and "vmcnt" in i:
+                    run = 0
+            assert longest >= 8, (name, longest)     # the compiler may start folding before the ninth
 
 
 def test_float_min_max_stay_compare_select(asm):

@@ -38,6 +38,15 @@ std::atomic<int> g_resident{0};
 std::atomic<int> g_tail_flag{1};
 std::atomic<unsigned> g_shape_epoch{0}; // bumped when a launch-shape knob changes
 std::atomic<unsigned> g_max_counted_grid{2048}; // measured (blocking call, us, counting / queued kernel): 512 workgroups 8.0 / 9.2, 2048: 8.6-9.7 / 9.4-9.5, 8192: 10.4 / 10.0
+// Launches of at most this many workgroups (and at least 4 sources; up to 3 the
+// walk has every load in flight anyway) use the burst kernel: all loads of a
+// tile at once.  Such a launch leaves the memory side idle and is bound by the
+// chain of load latencies, which the walk makes as long as half the source count.
+// Measured, blocking call, fp32 SUM, us (walk / burst): 8 sources x 1 KiB 6.73 / 6.51,
+// x 32 KiB 8.00 / 7.78, x 2 MiB 9.57 / 9.29, x 4 MiB 11.35 / 11.27, x 16 MiB 28.9 / 30.6;
+// 16 sources x 1 KiB 7.39 / 6.89, x 512 KiB 10.50 / 9.16, x 2 MiB 11.94 / 10.92,
+// x 4 MiB 16.45 / 18.14; 4 sources: equal up to 2 MiB, the walk ahead beyond.
+std::atomic<unsigned> g_burst_max_grid{2048};
 std::atomic<int> g_cu_count[kMaxDevices];
 
 void read_env_once()
@@ -49,6 +58,10 @@ void read_env_once()
     const char *res = getenv("XCCL_MC_ROCM_RESIDENT_PER_CU");
     const char *tf  = getenv("XCCL_MC_ROCM_TAIL_FLAG");
     g_tail_flag.store(tf ? atoi(tf) != 0 : 1, std::memory_order_release);
+    const char *bmg = getenv("XCCL_MC_ROCM_BURST_MAX_GRID");
+    if (bmg != nullptr && atoi(bmg) >= 0) {
+        g_burst_max_grid.store((unsigned)atoi(bmg), std::memory_order_release);
+    }
     const char *mcg = getenv("XCCL_MC_ROCM_MAX_COUNTED_GRID");
     if (mcg != nullptr && atoi(mcg) >= 0 && (unsigned)atoi(mcg) <= kMaxFlaggedGrid) {
         g_max_counted_grid.store((unsigned)atoi(mcg), std::memory_order_release);
@@ -151,7 +164,10 @@ unsigned lds_for_resident(uint32_t nsrc, size_t grid, int cus, size_t footprint)
 {
     int cap = g_resident.load(std::memory_order_relaxed);
     if (cap == 0) {
-        cap = (nsrc <= 2 || footprint <= ((size_t)192 << 20)) ? kNoResidentCap : nsrc == 3 ? 20 : 16;
+        // 8 and more sources want the bound from 8 MiB vectors on (16 sources x 8 MiB: 6.85 TB/s against
+        // 6.36 without, 8 x 8 MiB: 6.62 against 6.46), fewer sources only once the call outgrows the cache
+        const size_t fits = (size_t)(nsrc >= 8 ? 64 : 192) << 20;
+        cap = (nsrc <= 2 || footprint <= fits) ? kNoResidentCap : nsrc == 3 ? 20 : 16;
     }
     if (cap >= kNoResidentCap || grid <= (size_t)cap * (size_t)cus) {
         return 0; // the whole grid is resident at once anyway
@@ -246,7 +262,7 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     }
     plan->grid      = (unsigned)grid;
     plan->lds_bytes = lds_for_resident(nsrc, grid, cus, (size_t)(nsrc + 1) * elems * esize);
-    plan->fn        = e->fn;
+    plan->fn        = (nsrc >= 4 && grid <= g_burst_max_grid.load(std::memory_order_relaxed)) ? e->fn_burst : e->fn;
     return XCCL_OK;
 }
 
@@ -551,14 +567,11 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
         return st;
     }
     // Who writes the completion word: the launch itself, counting its workgroups (cheapest for small
-    // grids), or a one-lane kernel queued behind it (cheaper from about a thousand workgroups on).  The
-    // second needs every result store of the launch to be a write-through vector store: those are in
-    // memory when the reduction kernel ends, while peeled head/tail elements may sit dirty in an L2 until
-    // the runtime's own release at a stream synchronisation -- such launches count up to the larger bound
-    // and beyond it complete through the stream.
+    // grids), or a one-lane kernel queued behind it (cheaper from a few thousand workgroups on).  The
+    // second relies on every result store of the reduction being a write-through store: those are in
+    // memory when the reduction kernel ends, and stream order starts the one-lane kernel after that.
     const bool     want_flag = dev_count != nullptr && dev_flag != nullptr && flagged != nullptr;
-    const bool     tail_ok   = want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0 &&
-                               plan.args.head + plan.args.tail == 0;
+    const bool     tail_ok   = want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0;
     const unsigned counted   = tail_ok ? g_max_counted_grid.load(std::memory_order_relaxed) : kMaxFlaggedGrid;
     const bool     in_kernel = want_flag && plan.grid <= counted;
     if (in_kernel) {
@@ -686,6 +699,13 @@ void xccl_rocm_set_launch_shape(int blocks_per_cu, int resident_per_cu)
     g_resident.store(resident_per_cu > 0 ? resident_per_cu : 0, std::memory_order_release);
     g_blocks_per_cu.store(blocks_per_cu > 0 ? blocks_per_cu : kDefaultBlocksPerCu, std::memory_order_release);
     g_shape_epoch.fetch_add(1, std::memory_order_release); // plans cached by the threads are stale now
+}
+
+void xccl_rocm_set_burst_max_grid(int max_grid)
+{
+    read_env_once();
+    g_burst_max_grid.store(max_grid >= 0 ? (unsigned)max_grid : 2048u, std::memory_order_release);
+    g_shape_epoch.fetch_add(1, std::memory_order_release);
 }
 
 xccl_status_t xccl_rocm_reduce_multi_plan(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,

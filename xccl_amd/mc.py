@@ -95,6 +95,8 @@ def component_lib():
         lib.xccl_rocm_graph_cache_destroy.restype = None
         lib.xccl_rocm_set_launch_shape.argtypes = [_int, _int]
         lib.xccl_rocm_set_launch_shape.restype = None
+        lib.xccl_rocm_set_burst_max_grid.argtypes = [_int]
+        lib.xccl_rocm_set_burst_max_grid.restype = None
         _u32p = _c.POINTER(_c.c_uint32)
         lib.xccl_rocm_reduce_multi_flagged.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp, _vp, _vp,
                                                        _c.c_uint32, _c.POINTER(_int)]
@@ -325,6 +327,16 @@ def bench_kernel_times(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, iters
     for e in evs:
         hip.event_destroy(e)
     return _st(st), out
+
+
+def reduce_multi_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op):
+    """What a launch with these arguments would be: mangled kernel name, grid and block size."""
+    grid, block, name = _c.c_uint(0), _c.c_uint(0), _c.create_string_buffer(256)
+    st = component_lib().xccl_rocm_reduce_multi_plan(sbuf1, sbuf2, rbuf, count, size, stride, int(dtype), int(op),
+                                                     _c.byref(grid), _c.byref(block), name, 256)
+    if _st(st) != Status.OK:
+        raise RuntimeError("xccl_rocm_reduce_multi_plan: %s" % _st(st))
+    return {"kernel": name.value.decode(), "grid": grid.value, "block": block.value}
 
 
 def bench_region_time_rot(sbuf1, sbuf2, rbuf, rot_count, rot_pitch, count, size, stride, dtype, op, iters: int):
