@@ -92,6 +92,32 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
                                              int *flagged);
 
 /*
+ * xccl_rocm_reduce_multi_flagged for a caller whose completion word is the
+ * first of `flag_words` consecutive 32-bit words (host-mapped, device view in
+ * `dev_flag`).  A launch of 2 to 8 workgroups (XCCL_MC_ROCM_SLOT_MAX_GRID, at
+ * most min(flag_words, XCCL_ROCM_FLAG_WORDS)) then reports completion without
+ * any counting: workgroup b stores `seq` to dev_flag[b] once its own result
+ * stores are in memory, `*flagged` is set to the number of workgroups, and
+ * the launch is complete when the first `*flagged` words all hold `seq`
+ * (words beyond keep what earlier launches left there: compare for equality
+ * with a `seq` that differs from launch to launch).  That spares such a launch
+ * the round trip of an arrival atomic: blocking call, 2 sources x 2 KiB
+ * 6.8-7.1 -> 6.4 us, 8 sources x 8 KiB 7.6-7.9 -> 7.4-7.5 us; every further
+ * word costs the host's view about 0.1 us, so that from 12 workgroups on
+ * counting is as fast and from 16 on faster (2 x 16 KiB: 7.7 against 7.9 us).
+ * Every other launch behaves as under xccl_rocm_reduce_multi_flagged and sets
+ * `*flagged` to 1 or 0.  No counterpart in the reference.
+ */
+#define XCCL_ROCM_FLAG_WORDS 16
+xccl_status_t xccl_rocm_reduce_multi_slots(void *sbuf1, void *sbuf2, void *rbuf,
+                                           size_t count, size_t size,
+                                           size_t stride, xccl_dt_t dtype,
+                                           xccl_op_t op, void *hip_stream,
+                                           uint32_t *dev_count,
+                                           uint32_t *dev_flag, uint32_t flag_words,
+                                           uint32_t seq, int *flagged);
+
+/*
  * xccl_rocm_reduce_multi_flagged for callers that must not allocate: code
  * under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  It has no counterpart in the reference.  The arrival counters
@@ -162,6 +188,11 @@ void xccl_rocm_set_launch_shape(int blocks_per_cu, int resident_per_cu);
  * also XCCL_MC_ROCM_BURST_MAX_GRID.  For measurement and tests.
  */
 void xccl_rocm_set_burst_max_grid(int max_grid);
+
+/* Largest launch, in workgroups, that reports completion on one word per
+ * workgroup (xccl_rocm_reduce_multi_slots); 0 = never, negative = the built-in
+ * default (8).  For measurement and tests. */
+void xccl_rocm_set_slot_max_grid(int max_grid);
 
 /* What a launch with these arguments would be: grid/block size and the
  * mangled kernel name (truncated into `name`, if not NULL).  Host-only apart

@@ -391,6 +391,92 @@ def test_completion_word_threshold_and_sequences(rocm, oracle):
         c.close()
 
 
+def test_completion_by_one_word_per_workgroup(rocm, oracle):
+    """Launches of a handful of workgroups (2 to 8 by default, up to 16 on
+    request) report completion without counting: workgroup b stores the
+    sequence number to word b of the caller's 16 words.  Through the C ABI:
+    the number of words to watch comes back in `flagged`, each of them ends up
+    holding the sequence number, words beyond keep what they held, and the
+    result is the oracle's; a caller with too few words, a launch of one
+    workgroup and one beyond the bound get the counting path (`flagged` 1).
+    Then the same shapes through the component's blocking entry and
+    reduce_multi_nb + event_query, with the path switched off and on."""
+    lib = rocm.component_lib()
+    stream = rocm.component_stream()
+    words = 16
+    host = hip.host_malloc(4 * words)
+    ctypes.memset(host, 0, 4 * words)
+    dev = hip.host_get_device_pointer(host)
+    view = ctypes.cast(host, ctypes.POINTER(ctypes.c_uint32))
+    counters = hip.malloc((1 + 64) * 128)
+    hip.memset(counters, 0, (1 + 64) * 128)
+    hip.device_synchronize()
+    dt, op, n2 = Dt.FLOAT32, Op.SUM, 3
+    seq = 0
+    try:
+        for bound, tiles, room, expect_words in ((-1, 1, 16, 1), (-1, 2, 16, 2), (-1, 7, 16, 7), (-1, 8, 16, 8),
+                                                 (-1, 9, 16, 1), (16, 9, 16, 9), (16, 16, 16, 16), (16, 17, 16, 1),
+                                                 (64, 17, 64, 1), (-1, 7, 1, 1), (-1, 7, 4, 1), (-1, 4, 4, 4),
+                                                 (0, 4, 16, 1)):
+            lib.xccl_rocm_set_slot_max_grid(bound)
+            size = tiles * 256 - 3              # ragged last tile, peeled tail elements
+            c = Case(dt, size, n2)
+            try:
+                c.fill_random(oracle, 90 + tiles)
+                c.upload()
+                p1, p2, pr = c.ptrs()
+                want, _ = c.expect(oracle, op)
+                hip.memset(pr, 0xAB, c.vbytes)
+                hip.device_synchronize()
+                before = [view[i] for i in range(words)]
+                seq += 1
+                flagged = ctypes.c_int(-1)
+                st = lib.xccl_rocm_reduce_multi_slots(p1, p2, pr, n2, size, c.stride, int(dt), int(op), stream, counters,
+                                                      dev, room, seq, ctypes.byref(flagged))
+                assert st == Status.OK
+                assert flagged.value == expect_words, (tiles, room, flagged.value)
+                t0 = time.time()
+                while any(view[i] != seq for i in range(flagged.value)):
+                    assert time.time() - t0 < 20.0, "completion words never written: %s" % [view[i] for i in range(8)]
+                assert_same(c.result(), want, dt, op, "%d tiles, room for %d words" % (tiles, room))
+                hip.stream_synchronize(stream)
+                assert [view[i] for i in range(flagged.value, words)] == before[flagged.value:], (tiles, room)
+            finally:
+                c.close()
+        for max_grid in (0, -1, 16):
+            lib.xccl_rocm_set_slot_max_grid(max_grid)
+            for tiles in (2, 3, 7, 8, 9, 16, 17):
+                size = tiles * 256 - 1
+                c = Case(dt, size, n2)
+                try:
+                    c.fill_random(oracle, 190 + tiles)
+                    c.upload()
+                    p1, p2, pr = c.ptrs()
+                    want, _ = c.expect(oracle, op)
+                    for rep in range(3):
+                        hip.memset(pr, 0x10 + rep, c.vbytes)
+                        assert rocm.xccl_mem_component_reduce_multi(p1, p2, pr, n2, size, c.stride, dt, op,
+                                                                    MemType.ROCM) == Status.OK
+                        assert_same(c.result(), want, dt, op, "blocking, %d tiles, rep %d" % (tiles, rep))
+                        hip.memset(pr, 0x20 + rep, c.vbytes)
+                        st, ev = rocm.xccl_mem_component_reduce_multi_nb(p1, p2, pr, n2, size, c.stride, dt, op,
+                                                                         MemType.ROCM, None)
+                        assert st == Status.OK and ev is not None
+                        t0 = time.time()
+                        while rocm.xccl_mc_event_query(ev) == Status.INPROGRESS:
+                            assert time.time() - t0 < 20.0
+                        assert rocm.xccl_mc_event_query(ev) == Status.OK
+                        assert_same(c.result(), want, dt, op, "event, %d tiles, rep %d" % (tiles, rep))
+                        assert rocm.xccl_mc_event_free(ev) == Status.OK
+                finally:
+                    c.close()
+    finally:
+        lib.xccl_rocm_set_slot_max_grid(-1)
+        hip.stream_synchronize(stream)
+        hip.free(counters)
+        hip.host_free(host)
+
+
 def test_many_events_in_flight_any_wait_order(rocm, oracle):
     """One pooled event per launch, 48 launches enqueued before the first wait,
     waited for in reverse order, mixed small (completion word) and large

@@ -72,14 +72,15 @@ def test_completion_word_waits_for_the_result_stores(asm):
             stores = [m.start() for m in re.finditer(r"\bbuffer_store_\w+\b", body)]
             atomics = [m.start() for m in re.finditer(r"\bglobal_atomic_inc\b", body)]
             publish = [m.start() for m in re.finditer(r"\bglobal_store_dword\b[^\n]* sc0 sc1", body)]
-            assert stores and len(atomics) == 2 and len(publish) == 1, (name, len(stores), len(atomics), len(publish))
+            # two publishing stores: one word per workgroup for a handful of workgroups, the counted path's last arriver
+            assert stores and len(atomics) == 2 and len(publish) == 2, (name, len(stores), len(atomics), len(publish))
             assert max(stores) < wait < min(atomics + publish), name
             # nothing branches from the tile loop to behind the wait: the label the loop exits to precedes it
             assert not re.search(r"\bbuffer_(load|store)_\w+\b", body[wait:]), name
-            # every result store is a buffer store with write-through policy: the publishing store (a system-scope
-            # release, which brings the kernel's only cache write-back) is the only global/flat store
-            assert len(re.findall(r"\b(global|flat)_store_\w+", body)) == 1, name
-            assert body.count("buffer_wbl2") == 1, name
+            # every result store is a buffer store with write-through policy: the publishing stores (system-scope
+            # releases, which bring the kernel's only cache write-backs) are the only global/flat stores
+            assert len(re.findall(r"\b(global|flat)_store_\w+", body)) == 2, name
+            assert body.count("buffer_wbl2") == 2, name
 
 
 def test_code_generation_properties(asm):

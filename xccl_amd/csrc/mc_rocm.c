@@ -71,7 +71,7 @@ typedef struct mc_rocm_event {
     xccl_mc_event_t    super;
     atomic_int         is_free;
     hipEvent_t         hip_event;
-    int                flagged;   /* 1: done when *flag == expect */
+    int                flagged;   /* n > 0: done when the first n words at flag all equal expect */
     uint32_t           expect;    /* last sequence number handed to a kernel */
     volatile uint32_t *flag;      /* host view of the completion word */
     uint32_t          *dev_flag;  /* device view of the same word */
@@ -89,7 +89,10 @@ typedef struct mc_rocm_event {
 #define MC_CPU_RELAX() ((void)0)
 #endif
 
-#define MC_FLAG_STRIDE 16 /* uint32 words between completion words: one per 64-byte line */
+/* uint32 words per event, one 64-byte line: a launch of a handful of workgroups
+ * reports on one word per workgroup (xccl_rocm_reduce_multi_slots), every
+ * other on the first */
+#define MC_FLAG_STRIDE XCCL_ROCM_FLAG_WORDS
 
 typedef struct mc_rocm_stream_request {
     xccl_mem_component_stream_request_t super;
@@ -429,6 +432,19 @@ static xccl_status_t mc_rocm_mem_type(void *ptr, ucs_memory_type_t *mem_type)
     return XCCL_OK;
 }
 
+/* Whether the flagged launch an event stands for has completed. */
+static int mc_rocm_flag_done(const mc_rocm_event_t *ev)
+{
+    int i;
+
+    for (i = 0; i < ev->flagged; i++) {
+        if (__atomic_load_n(&ev->flag[i], __ATOMIC_ACQUIRE) != ev->expect) {
+            return 0;
+        }
+    }
+    return 1;
+}
+
 static mc_rocm_event_t *mc_rocm_claim_event(mc_rocm_device_t *d)
 {
     /* threads start their search in different quarters of the pool, so that
@@ -442,7 +458,7 @@ static mc_rocm_event_t *mc_rocm_claim_event(mc_rocm_device_t *d)
         if (!atomic_compare_exchange_strong(&ev->is_free, &expect, MC_SLOT_BUSY)) {
             continue;
         }
-        if (ev->flagged && __atomic_load_n(ev->flag, __ATOMIC_ACQUIRE) != ev->expect) {
+        if (ev->flagged && !mc_rocm_flag_done(ev)) {
             /* freed by its owner before the launch it stands for finished: its
              * completion word and arrival counter are still in use */
             atomic_store(&ev->is_free, MC_SLOT_FREE);
@@ -470,14 +486,13 @@ static xccl_status_t mc_rocm_flag_poll(mc_rocm_event_t *ev, int block)
     hipError_t e;
 
     for (;;) {
-        if (__atomic_load_n(ev->flag, __ATOMIC_ACQUIRE) == ev->expect) {
+        if (mc_rocm_flag_done(ev)) {
             return XCCL_OK;
         }
         if ((++ev->polls & 0xffffu) == 0) {
             e = hipStreamQuery(ev->stream);
             if (e == hipSuccess) {
-                return __atomic_load_n(ev->flag, __ATOMIC_ACQUIRE) == ev->expect
-                           ? XCCL_OK : XCCL_ERR_NO_MESSAGE;
+                return mc_rocm_flag_done(ev) ? XCCL_OK : XCCL_ERR_NO_MESSAGE;
             }
             if (e != hipErrorNotReady) {
                 return XCCL_ERR_NO_MESSAGE;
@@ -539,10 +554,11 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
         st = xccl_rocm_reduce_multi_graph(sbuf1, sbuf2, rbuf, count, size,
                                           stride, dtype, op, hs);
     } else if (ev != NULL) {
-        st = xccl_rocm_reduce_multi_flagged(sbuf1, sbuf2, rbuf, count, size,
-                                            stride, dtype, op, hs,
-                                            ev->dev_count, ev->dev_flag,
-                                            ev->expect + 1, &flagged);
+        st = xccl_rocm_reduce_multi_slots(sbuf1, sbuf2, rbuf, count, size,
+                                          stride, dtype, op, hs,
+                                          ev->dev_count, ev->dev_flag,
+                                          MC_FLAG_STRIDE, ev->expect + 1,
+                                          &flagged);
     } else {
         st = xccl_rocm_reduce_multi_impl(sbuf1, sbuf2, rbuf, count, size,
                                          stride, dtype, op, hs);

@@ -67,6 +67,7 @@ struct ReduceArgs {
     // is through, done_seq is stored to *done_flag, a host-mapped word the caller polls.
     uint32_t    done_seq;
     uint32_t   *done_count; // device words (1 + kDoneShards, kDoneStride apart), zero between launches
+    uint32_t    done_slots; // != 0: no counting, workgroup b stores done_seq to done_flag[b] (grid <= done_slots)
     uint32_t   *done_flag;
 };
 
@@ -357,6 +358,15 @@ __device__ __forceinline__ void fold_tile_burst(const ReduceArgs &a, size_t v0)
 __device__ __forceinline__ void publish_completion(const ReduceArgs &a)
 {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (a.done_slots != 0) {
+        // A handful of workgroups: each reports on a word of its own and the host
+        // looks at all of them, which spares the launch the round trip of an
+        // arrival atomic and the arrivals their turn on one counter.
+        if (threadIdx.x == 0) {
+            __hip_atomic_store(a.done_flag + blockIdx.x, a.done_seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        return;
+    }
     if (threadIdx.x == 0) {
         // Arrival counting in two levels, so that no single word takes more than
         // grid/kDoneShards increments: workgroup b counts into shard b % shards, the

@@ -47,6 +47,10 @@ std::atomic<unsigned> g_max_counted_grid{2048}; // measured (blocking call, us, 
 // 16 sources x 1 KiB 7.39 / 6.89, x 512 KiB 10.50 / 9.16, x 2 MiB 11.94 / 10.92,
 // x 4 MiB 16.45 / 18.14; 4 sources: equal up to 2 MiB, the walk ahead beyond.
 std::atomic<unsigned> g_burst_max_grid{2048};
+// Launches of at most this many workgroups report completion on one word per
+// workgroup when the caller has room for them (see xccl_rocm_reduce_multi_slots).
+constexpr unsigned kDefaultSlotMaxGrid = 8; // measured: see xccl_rocm_reduce_multi_slots in the header
+std::atomic<unsigned> g_slot_max_grid{kDefaultSlotMaxGrid};
 std::atomic<int> g_cu_count[kMaxDevices];
 
 void read_env_once()
@@ -61,6 +65,10 @@ void read_env_once()
     const char *bmg = getenv("XCCL_MC_ROCM_BURST_MAX_GRID");
     if (bmg != nullptr && atoi(bmg) >= 0) {
         g_burst_max_grid.store((unsigned)atoi(bmg), std::memory_order_release);
+    }
+    const char *smg = getenv("XCCL_MC_ROCM_SLOT_MAX_GRID");
+    if (smg != nullptr && atoi(smg) >= 0) {
+        g_slot_max_grid.store((unsigned)atoi(smg), std::memory_order_release);
     }
     const char *mcg = getenv("XCCL_MC_ROCM_MAX_COUNTED_GRID");
     if (mcg != nullptr && atoi(mcg) >= 0 && (unsigned)atoi(mcg) <= kMaxFlaggedGrid) {
@@ -182,6 +190,7 @@ bool same_plan(const Plan &a, const Plan &b)
            a.args.dst == b.args.dst && a.args.stride == b.args.stride && a.args.head == b.args.head &&
            a.args.nvec == b.args.nvec && a.args.tail == b.args.tail && a.args.n2 == b.args.n2 &&
            a.args.done_flag == b.args.done_flag && a.args.done_count == b.args.done_count &&
+           a.args.done_slots == b.args.done_slots &&
            a.args.done_seq == b.args.done_seq;
 }
 
@@ -251,6 +260,7 @@ xccl_status_t make_plan(void *s1, void *s2, void *dst, size_t count, size_t size
     a.n2     = n2;
     a.done_seq   = 0;
     a.done_count = nullptr;
+    a.done_slots = 0;
     a.done_flag  = nullptr;
 
     const size_t tile  = (size_t)kBlock;
@@ -557,6 +567,15 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
                                              size_t stride, xccl_dt_t dtype, xccl_op_t op, void *hip_stream,
                                              uint32_t *dev_count, uint32_t *dev_flag, uint32_t seq, int *flagged)
 {
+    return xccl_rocm_reduce_multi_slots(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, hip_stream, dev_count,
+                                        dev_flag, 1, seq, flagged);
+}
+
+xccl_status_t xccl_rocm_reduce_multi_slots(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
+                                           size_t stride, xccl_dt_t dtype, xccl_op_t op, void *hip_stream,
+                                           uint32_t *dev_count, uint32_t *dev_flag, uint32_t flag_words, uint32_t seq,
+                                           int *flagged)
+{
     if (flagged) {
         *flagged = 0;
     }
@@ -574,16 +593,21 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
     const bool     tail_ok   = want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0;
     const unsigned counted   = tail_ok ? g_max_counted_grid.load(std::memory_order_relaxed) : kMaxFlaggedGrid;
     const bool     in_kernel = want_flag && plan.grid <= counted;
+    // a grid of one needs neither counting nor a second word: it stays on the counting path, which then has no atomics
+    const unsigned slots_max = flag_words < XCCL_ROCM_FLAG_WORDS ? flag_words : XCCL_ROCM_FLAG_WORDS;
+    const bool     by_slots  = in_kernel && plan.grid > 1 && plan.grid <= slots_max &&
+                               plan.grid <= g_slot_max_grid.load(std::memory_order_relaxed);
     if (in_kernel) {
         plan.args.done_seq   = seq;
         plan.args.done_count = dev_count;
+        plan.args.done_slots = by_slots ? plan.grid : 0;
         plan.args.done_flag  = dev_flag;
     }
     void *argv[1] = {&plan.args};
     HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, plan.lds_bytes,
                                 (hipStream_t)hip_stream));
     if (in_kernel) {
-        *flagged = 1;
+        *flagged = by_slots ? (int)plan.grid : 1;
     } else if (tail_ok) {
         hipLaunchKernelGGL(tail_flag_kernel, dim3(1), dim3(1), 0, (hipStream_t)hip_stream, dev_flag, seq);
         if (hipGetLastError() == hipSuccess) {
@@ -699,6 +723,13 @@ void xccl_rocm_set_launch_shape(int blocks_per_cu, int resident_per_cu)
     g_resident.store(resident_per_cu > 0 ? resident_per_cu : 0, std::memory_order_release);
     g_blocks_per_cu.store(blocks_per_cu > 0 ? blocks_per_cu : kDefaultBlocksPerCu, std::memory_order_release);
     g_shape_epoch.fetch_add(1, std::memory_order_release); // plans cached by the threads are stale now
+}
+
+void xccl_rocm_set_slot_max_grid(int max_grid)
+{
+    read_env_once();
+    g_slot_max_grid.store(max_grid >= 0 ? (unsigned)max_grid : kDefaultSlotMaxGrid, std::memory_order_release);
+    g_shape_epoch.fetch_add(1, std::memory_order_release);
 }
 
 void xccl_rocm_set_burst_max_grid(int max_grid)

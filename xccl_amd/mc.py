@@ -97,6 +97,10 @@ def component_lib():
         lib.xccl_rocm_set_launch_shape.restype = None
         lib.xccl_rocm_set_burst_max_grid.argtypes = [_int]
         lib.xccl_rocm_set_burst_max_grid.restype = None
+        lib.xccl_rocm_set_slot_max_grid.argtypes = [_int]
+        lib.xccl_rocm_set_slot_max_grid.restype = None
+        lib.xccl_rocm_reduce_multi_slots.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp, _vp, _vp,
+                                                     _c.c_uint32, _c.c_uint32, _c.POINTER(_int)]
         _u32p = _c.POINTER(_c.c_uint32)
         lib.xccl_rocm_reduce_multi_flagged.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp, _vp, _vp,
                                                        _c.c_uint32, _c.POINTER(_int)]
