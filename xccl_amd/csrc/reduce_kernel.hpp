@@ -27,6 +27,10 @@
 // The launch asks for LDS it never touches to hold the resident workgroups
 // per compute unit to 16-32 (by source count): the memory side saturates
 // before the wave slots do.
+//   Launches of a few thousand tiles at most are a different regime: the
+// memory side is idle and the call is bound by the chain of load latencies.
+// They run the second form of the kernel (Burst = true), which does issue
+// the loads of up to nine sources at once.
 //
 // Layout of one call, in elements of T:
 //     [0, head)                 peeled so that the vector body starts on a
