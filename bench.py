@@ -171,6 +171,16 @@ def latency_sweep(mc, hip, iters, quick):
                 ns = ns[n // 10:]
                 row[mode] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
                              "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
+            # the blocking entry once more with the component's own dispatch queue switched off: the same launch
+            # through hipLaunchKernel on the component's stream
+            mc.component_lib().xccl_rocm_set_direct_queue(0)
+            st, ns = mc.bench_latency("sync", buf.ptr, buf.ptr + maxb, buf.ptr + 9 * maxb, nsrc - 1, cnt, maxb,
+                                      Dt.FLOAT32, Op.SUM, iters)
+            mc.component_lib().xccl_rocm_set_direct_queue(1)
+            assert st == Status.OK, st
+            ns = ns[iters // 10:]
+            row["sync_on_hip_stream"] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
+                                         "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
             res["n%d_%dB" % (nsrc, b)] = row
     # where the time of a one-node graph launch goes (4 sources x 1 KiB, completion word carried by the graph)
     st, parts = mc.bench_graph_parts(buf.ptr, buf.ptr + maxb, buf.ptr + 9 * maxb, 3, 256, maxb, Dt.FLOAT32, Op.SUM, 3000)

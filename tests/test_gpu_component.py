@@ -477,6 +477,61 @@ def test_completion_by_one_word_per_workgroup(rocm, oracle):
         hip.host_free(host)
 
 
+def test_blocking_calls_take_the_components_own_queue(rocm, oracle):
+    """A blocking reduction small enough to carry its completion word goes out
+    on the component's own dispatch queue, not on a HIP stream -- unless the
+    path is switched off, the call is too large, or the calling thread has
+    stream-ordered launches outstanding that the call has to stay behind.
+    The counter of such launches says which way a call went; the result is
+    the oracle's every time."""
+    lib = rocm.component_lib()
+    dt, op, n2 = Dt.FLOAT32, Op.SUM, 3
+    small, large = Case(dt, 5000, n2), Case(dt, 3 * 1024 * 1024, n2)
+
+    def blocking(c, tag):
+        p1, p2, pr = c.ptrs()
+        hip.memset(pr, 0x5C, c.vbytes)
+        hip.device_synchronize()
+        before = lib.xccl_rocm_direct_launch_count()
+        assert rocm.xccl_mem_component_reduce_multi(p1, p2, pr, n2, c.size, c.stride, dt, op, MemType.ROCM) == Status.OK
+        assert_same(c.result(), c.expect(oracle, op)[0], dt, op, tag)
+        return lib.xccl_rocm_direct_launch_count() - before
+
+    try:
+        for c in (small, large):
+            c.fill_random(oracle, 33)
+            c.upload()
+        blocking(small, "whichever way: earlier tests may have left stream-ordered launches nobody waited for")
+        assert blocking(small, "own queue") == 1
+        assert blocking(small, "own queue again") == 1
+        assert blocking(large, "12 MiB vectors: the stream") == 0
+        lib.xccl_rocm_set_direct_queue(0)
+        assert blocking(small, "switched off") == 0
+        lib.xccl_rocm_set_direct_queue(1)
+        # a stream-ordered launch nobody has waited for: the next blocking call stays behind it on the stream
+        p1, p2, pr = large.ptrs()
+        st, ev = rocm.xccl_mem_component_reduce_multi_nb(p1, p2, pr, n2, large.size, large.stride, dt, op, MemType.ROCM,
+                                                         None)
+        assert st == Status.OK and ev is not None
+        assert blocking(small, "behind a stream-ordered launch") == 0
+        assert rocm.xccl_mc_event_query(ev) == Status.OK        # stream order: it has completed as well
+        assert rocm.xccl_mc_event_free(ev) == Status.OK
+        assert_same(large.result(), large.expect(oracle, op)[0], dt, op, "the stream-ordered launch")
+        assert blocking(small, "own queue once the stream has been waited for") == 1
+        # 2000 in a row: kernel-argument slots and packets are reused many times over
+        p1, p2, pr = small.ptrs()
+        before = lib.xccl_rocm_direct_launch_count()
+        for rep in range(2000):
+            assert rocm.xccl_mem_component_reduce_multi(p1, p2, pr, n2, small.size, small.stride, dt, op,
+                                                        MemType.ROCM) == Status.OK
+        assert lib.xccl_rocm_direct_launch_count() - before == 2000
+        assert_same(small.result(), small.expect(oracle, op)[0], dt, op, "after 2000 calls")
+    finally:
+        lib.xccl_rocm_set_direct_queue(1)
+        small.close()
+        large.close()
+
+
 def test_many_events_in_flight_any_wait_order(rocm, oracle):
     """One pooled event per launch, 48 launches enqueued before the first wait,
     waited for in reverse order, mixed small (completion word) and large

@@ -243,6 +243,26 @@ def test_walk_and_burst_kernels_agree_with_the_oracle(rocm, oracle):
         lib.xccl_rocm_set_burst_max_grid(-1)
 
 
+def test_every_dtype_op_on_the_stream_path(rocm, oracle):
+    """Blocking calls normally go out on the component's own dispatch queue,
+    whose kernels are loaded from code objects embedded in the library; with
+    that path switched off the same calls run the kernels of the HIP module on
+    a HIP stream.  Every supported (dtype, op), both kernel forms."""
+    lib = rocm.component_lib()
+    try:
+        lib.xccl_rocm_set_direct_queue(0)
+        before = lib.xccl_rocm_direct_launch_count()
+        for i, (dt, op) in enumerate(supported_pairs()):
+            run_and_check(rocm, oracle, dt, op, 2000 + 11 * i, (1, 2, 5, 9)[i % 4], seed=500 + i)
+        assert lib.xccl_rocm_direct_launch_count() == before
+        lib.xccl_rocm_set_direct_queue(1)       # (the calls above were blocking: nothing is left on the stream)
+        for i, (dt, op) in enumerate(supported_pairs()):
+            run_and_check(rocm, oracle, dt, op, 2000 + 11 * i, (1, 2, 5, 9)[i % 4], seed=500 + i)
+        assert lib.xccl_rocm_direct_launch_count() - before == len(supported_pairs())
+    finally:
+        lib.xccl_rocm_set_direct_queue(1)
+
+
 def test_randomised_shapes(rocm, oracle):
     """400 reproducible random calls: any supported (dtype, op), 1..20 vectors
     in sbuf2, sizes up to a few tiles, independent byte placement of the three

@@ -100,6 +100,9 @@ def test_code_generation_properties(asm):
                 all(i.endswith(" sc0 sc1") for i in stores), name
             # head and tail elements take the same route: no global/flat loads of operands at all
             assert not re.search(r"\b(global|flat)_load_(u?byte|u?short|dword)", body), name
+            # the kernel argument block is ReduceArgs and nothing else (no implicit launch arguments): the
+            # component's own dispatch queue passes exactly that
+            assert re.search(r"\.amdhsa_kernarg_size 96\b", body), name
             # few registers: 24 or more waves fit a compute unit
             assert int(re.search(r"\.amdhsa_next_free_vgpr (\d+)", body).group(1)) <= 80, name
 

@@ -22,6 +22,9 @@
  *   - freed device blocks are cached for the next mem_alloc (mc_pool.h);
  *   - small launches report completion through a host-mapped word the kernel
  *     writes itself, which the host sees sooner than the queue's signal;
+ *   - blocking reductions that complete through that word are launched on a
+ *     dispatch queue of the component's own (xccl_rocm_reduce_multi_direct),
+ *     not through hipLaunchKernel on a stream;
  *   - the vtable is extended with stream-ordered reductions whose completion
  *     is an event (see include/xccl_rocm_mem_component.h).
  *
@@ -77,6 +80,7 @@ typedef struct mc_rocm_event {
     uint32_t          *dev_flag;  /* device view of the same word */
     uint32_t          *dev_count; /* arrival counters of the launch's workgroups */
     hipStream_t        stream;    /* where the work was enqueued */
+    int                direct;    /* 1: launched on the component's own dispatch queue, not on `stream` */
     unsigned           polls;
 } mc_rocm_event_t;
 
@@ -108,6 +112,9 @@ typedef struct mc_rocm_device {
     int                     *gate_words;  /* pinned, mapped */
     uint32_t                *flag_words; /* pinned, mapped: completion words of the events */
     uint32_t                *arrival_counts; /* device */
+    /* nonzero while a reduction stream may hold stream-ordered launches nobody has waited for: a blocking
+     * call of that slot then stays on the stream, behind them, instead of taking the dispatch queue */
+    atomic_int               unsynced[MC_NUM_STREAMS];
     mc_rocm_event_t          events[XCCL_ROCM_MC_NUM_EVENTS];
     mc_rocm_stream_request_t requests[XCCL_ROCM_MC_NUM_STREAM_REQUESTS];
 } mc_rocm_device_t;
@@ -335,9 +342,14 @@ static unsigned mc_rocm_thread_index(void)
     return (unsigned)index;
 }
 
+static int mc_rocm_thread_slot(void)
+{
+    return (int)(mc_rocm_thread_index() % (unsigned)mc_num_streams);
+}
+
 static xccl_status_t mc_rocm_thread_stream(mc_rocm_device_t *d, hipStream_t *out)
 {
-    const int     slot = (int)(mc_rocm_thread_index() % (unsigned)mc_num_streams);
+    const int     slot = mc_rocm_thread_slot();
     xccl_status_t st   = XCCL_OK;
 
     if (__atomic_load_n(&d->stream[slot], __ATOMIC_ACQUIRE) == NULL) {
@@ -480,7 +492,8 @@ static xccl_status_t mc_rocm_user_stream(xccl_stream_t *stream, hipStream_t *out
 
 /* Completion of a flagged launch, observed from the host.  `block`: spin until
  * done.  Every 64 Ki polls the stream is asked whether it failed or drained
- * without the word being written, so a broken launch cannot spin forever. */
+ * without the word being written (a launch on the component's own queue: whether
+ * that queue reported an error), so a broken launch cannot spin forever. */
 static xccl_status_t mc_rocm_flag_poll(mc_rocm_event_t *ev, int block)
 {
     hipError_t e;
@@ -489,7 +502,11 @@ static xccl_status_t mc_rocm_flag_poll(mc_rocm_event_t *ev, int block)
         if (mc_rocm_flag_done(ev)) {
             return XCCL_OK;
         }
-        if ((++ev->polls & 0xffffu) == 0) {
+        if ((++ev->polls & 0xffffu) == 0 && ev->direct) {
+            if (xccl_rocm_direct_queue_failed()) {
+                return XCCL_ERR_NO_MESSAGE;
+            }
+        } else if ((ev->polls & 0xffffu) == 0) {
             e = hipStreamQuery(ev->stream);
             if (e == hipSuccess) {
                 return mc_rocm_flag_done(ev) ? XCCL_OK : XCCL_ERR_NO_MESSAGE;
@@ -550,6 +567,30 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
         }
     }
 
+    if (want_sync && stream == NULL && ev != NULL && mc_graph_max_bytes == 0 &&
+        atomic_load_explicit(&d->unsynced[mc_rocm_thread_slot()], memory_order_acquire) == 0) {
+        /* nothing of this thread's stream to stay behind, and the caller waits
+         * here: the launch needs no stream at all */
+        st = xccl_rocm_reduce_multi_direct(sbuf1, sbuf2, rbuf, count, size,
+                                           stride, dtype, op, mc_rocm_thread_slot(),
+                                           ev->dev_count, ev->dev_flag,
+                                           MC_FLAG_STRIDE, ev->expect + 1,
+                                           &flagged);
+        if (st == XCCL_OK && flagged) {
+            ev->stream  = hs;
+            ev->flagged = flagged;
+            ev->direct  = 1;
+            ev->polls   = 0;
+            ev->expect++;
+            st = mc_rocm_flag_poll(ev, 1);
+            atomic_store(&ev->is_free, MC_SLOT_FREE);
+            return st;
+        }
+        if (st != XCCL_OK) {
+            atomic_store(&ev->is_free, MC_SLOT_FREE);
+            return st;
+        }
+    }
     if (want_sync && size * xccl_dt_size(dtype) <= mc_graph_max_bytes) {
         st = xccl_rocm_reduce_multi_graph(sbuf1, sbuf2, rbuf, count, size,
                                           stride, dtype, op, hs);
@@ -569,9 +610,13 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
         }
         return st;
     }
+    if (stream == NULL && !want_sync) {
+        atomic_store_explicit(&d->unsynced[mc_rocm_thread_slot()], 1, memory_order_release);
+    }
     if (ev != NULL) {
         ev->stream  = hs;
         ev->flagged = flagged;
+        ev->direct  = 0;
         ev->polls   = 0;
         if (flagged) {
             ev->expect++;
@@ -585,6 +630,10 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
             st = mc_rocm_flag_poll(ev, 1);
         } else if (hipStreamSynchronize(hs) != hipSuccess) {
             st = XCCL_ERR_NO_MESSAGE;
+        }
+        if (stream == NULL && st == XCCL_OK) {
+            /* stream order: everything this slot's stream held before is complete as well */
+            atomic_store_explicit(&d->unsynced[mc_rocm_thread_slot()], 0, memory_order_release);
         }
     }
     if (ev != NULL) {
@@ -670,6 +719,7 @@ static xccl_status_t mc_rocm_event_record(xccl_stream_t *stream,
         return XCCL_ERR_NO_RESOURCE;
     }
     ev->flagged = 0;
+    ev->direct  = 0;
     ev->stream  = hs;
     e = hipEventRecord(ev->hip_event, hs);
     if (e != hipSuccess) {
@@ -865,6 +915,7 @@ static void mc_rocm_close(void)
             }
         }
         xccl_rocm_graph_cache_destroy();
+        xccl_rocm_direct_queue_destroy();
         mc_rocm_device_destroy(d); /* also clears `ready` */
     }
     (void)hipSetDevice(cur);

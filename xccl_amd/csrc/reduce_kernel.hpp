@@ -67,6 +67,7 @@ struct ReduceArgs {
     size_t      nvec;   // 16-byte vectors in the body
     size_t      tail;   // elements after the vector body
     uint32_t    n2;     // vectors in sbuf2 (>= 1)
+    uint32_t    grid;   // workgroups of the launch (the kernel reads no implicit launch arguments)
     // Completion word (small launches only; all NULL/0 otherwise): when the last workgroup
     // is through, done_seq is stored to *done_flag, a host-mapped word the caller polls.
     uint32_t    done_seq;
@@ -378,7 +379,7 @@ __device__ __forceinline__ void publish_completion(const ReduceArgs &a)
         // the last.  atomicInc wraps to zero at its bound, so every word is back at
         // zero by itself when the launch is over.  Words are kDoneStride apart
         // (one per 128-byte line): [0] top, [1 + s] shard s.
-        const uint32_t grid   = gridDim.x;
+        const uint32_t grid   = a.grid;
         const uint32_t shards = grid < kDoneShards ? grid : kDoneShards;
         bool           last   = true;
         if (grid > kDoneShards) {
@@ -402,7 +403,7 @@ template <typename T, class Op, bool Burst>
 __global__ void __launch_bounds__(kBlock) reduce_multi_kernel(const ReduceArgs a)
 {
     // Head and tail: one element per lane, by the last workgroup.
-    if (blockIdx.x == gridDim.x - 1) {
+    if (blockIdx.x == a.grid - 1) {
         if (a.head != 0) {
             fold_elements<T, Op>(a, -(ptrdiff_t)(a.head * sizeof(T)), (uint32_t)a.head);
         }
@@ -412,7 +413,7 @@ __global__ void __launch_bounds__(kBlock) reduce_multi_kernel(const ReduceArgs a
     }
     // One tile per workgroup in the usual launch; the loop only runs on when
     // there are more tiles than the grid cap allows workgroups.
-    const size_t step = (size_t)gridDim.x * kBlock;
+    const size_t step = (size_t)a.grid * kBlock;
     for (size_t v0 = (size_t)blockIdx.x * kBlock; v0 < a.nvec; v0 += step) {
         if (Burst) {
             fold_tile_burst<T, Op>(a, v0);

@@ -97,6 +97,10 @@ def component_lib():
         lib.xccl_rocm_set_launch_shape.restype = None
         lib.xccl_rocm_set_burst_max_grid.argtypes = [_int]
         lib.xccl_rocm_set_burst_max_grid.restype = None
+        lib.xccl_rocm_direct_launch_count.argtypes = []
+        lib.xccl_rocm_direct_launch_count.restype = _c.c_uint64
+        lib.xccl_rocm_set_direct_queue.argtypes = [_int]
+        lib.xccl_rocm_set_direct_queue.restype = None
         lib.xccl_rocm_set_slot_max_grid.argtypes = [_int]
         lib.xccl_rocm_set_slot_max_grid.restype = None
         lib.xccl_rocm_reduce_multi_slots.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp, _vp, _vp,
