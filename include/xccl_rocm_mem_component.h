@@ -99,10 +99,18 @@ extern "C" {
  *
  * reduce_nb / reduce_multi_nb: same arithmetic contract as reduce /
  * reduce_multi, but the call returns once the kernel is enqueued.
- *   stream == NULL : enqueue on the component's stream of the CALLING THREAD
+ *   stream == NULL : enqueue on the component's queue of the CALLING THREAD
  *                    (the one the synchronous entries use on that thread), so
  *                    successive calls of one thread are ordered among
- *                    themselves.  Threads are spread round-robin over up to 4
+ *                    themselves.  That queue is a HIP stream (get_stream) for
+ *                    calls without an event and for large ones; a call that
+ *                    has an event and is small enough to report its own
+ *                    completion goes out on a dispatch queue of the
+ *                    component's own instead when the stream holds nothing
+ *                    it would have to stay behind (5.2-6.6 us per call instead
+ *                    of 7.0-7.9; XCCL_MC_ROCM_DIRECT_QUEUE=0 switches that
+ *                    off).  The order of one thread's calls holds across the
+ *                    two; only the event tells when such a call is complete.  Threads are spread round-robin over up to 4
  *                    streams per device (XCCL_MC_ROCM_THREAD_STREAMS, 1..4),
  *                    so that blocking calls of several threads
  *                    (XCCL_THREAD_MODE_MULTIPLE) do not queue up behind each
@@ -149,7 +157,8 @@ typedef struct xccl_rocm_mem_component {
     xccl_status_t (*event_wait)(xccl_mc_event_t *event);
     /* The component's hipStream_t for the calling thread on the current
      * device (created on first use), as void*.  For callers that time or
-     * order work against it. */
+     * order work against it: calls of that thread with stream == NULL and
+     * event == NULL are on it; calls with an event may not be (above). */
     xccl_status_t (*get_stream)(void **hip_stream);
 } xccl_rocm_mem_component_t;
 

@@ -518,6 +518,27 @@ def test_blocking_calls_take_the_components_own_queue(rocm, oracle):
         assert rocm.xccl_mc_event_free(ev) == Status.OK
         assert_same(large.result(), large.expect(oracle, op)[0], dt, op, "the stream-ordered launch")
         assert blocking(small, "own queue once the stream has been waited for") == 1
+        # stream-ordered calls with an event take the own queue as well; a large one behind them goes to the
+        # stream after waiting for them on the host, so the order of one thread's calls holds across both
+        p1, p2, pr = small.ptrs()
+        hip.memset(pr, 0x3D, small.vbytes)
+        hip.device_synchronize()
+        before = lib.xccl_rocm_direct_launch_count()
+        st, ev_small = rocm.xccl_mem_component_reduce_multi_nb(p1, p2, pr, n2, small.size, small.stride, dt, op,
+                                                               MemType.ROCM, None)
+        assert st == Status.OK and ev_small is not None
+        assert lib.xccl_rocm_direct_launch_count() - before == 1
+        q1, q2, qr = large.ptrs()
+        st, ev_large = rocm.xccl_mem_component_reduce_multi_nb(q1, q2, qr, n2, large.size, large.stride, dt, op,
+                                                               MemType.ROCM, None)
+        assert st == Status.OK and ev_large is not None
+        assert rocm.xccl_mc_event_query(ev_small) == Status.OK      # the large launch was issued only after it
+        assert_same(small.result(), small.expect(oracle, op)[0], dt, op, "stream-ordered call on the own queue")
+        t0 = time.time()
+        while rocm.xccl_mc_event_query(ev_large) == Status.INPROGRESS:
+            assert time.time() - t0 < 20.0
+        assert rocm.xccl_mc_event_free(ev_small) == Status.OK and rocm.xccl_mc_event_free(ev_large) == Status.OK
+        assert blocking(small, "own queue: the large launch has been seen complete") == 1
         # 2000 in a row: kernel-argument slots and packets are reused many times over
         p1, p2, pr = small.ptrs()
         before = lib.xccl_rocm_direct_launch_count()

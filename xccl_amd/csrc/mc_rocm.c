@@ -81,6 +81,9 @@ typedef struct mc_rocm_event {
     uint32_t          *dev_count; /* arrival counters of the launch's workgroups */
     hipStream_t        stream;    /* where the work was enqueued */
     int                direct;    /* 1: launched on the component's own dispatch queue, not on `stream` */
+    int                slot;      /* reduction stream the launch went to, -1: a user's stream or the own queue */
+    unsigned           stream_seq; /* its number among the launches of that reduction stream */
+    struct mc_rocm_device *dev;
     unsigned           polls;
 } mc_rocm_event_t;
 
@@ -112,9 +115,11 @@ typedef struct mc_rocm_device {
     int                     *gate_words;  /* pinned, mapped */
     uint32_t                *flag_words; /* pinned, mapped: completion words of the events */
     uint32_t                *arrival_counts; /* device */
-    /* nonzero while a reduction stream may hold stream-ordered launches nobody has waited for: a blocking
-     * call of that slot then stays on the stream, behind them, instead of taking the dispatch queue */
-    atomic_int               unsynced[MC_NUM_STREAMS];
+    /* Launches put on each reduction stream, and the highest of them known to be complete (the stream runs
+     * them in order).  While the two differ, the stream may hold work nobody has waited for, and a call of that
+     * slot stays on the stream, behind it, instead of taking the component's own dispatch queue. */
+    atomic_uint              stream_issued[MC_NUM_STREAMS];
+    atomic_uint              stream_synced[MC_NUM_STREAMS];
     mc_rocm_event_t          events[XCCL_ROCM_MC_NUM_EVENTS];
     mc_rocm_stream_request_t requests[XCCL_ROCM_MC_NUM_STREAM_REQUESTS];
 } mc_rocm_device_t;
@@ -444,6 +449,65 @@ static xccl_status_t mc_rocm_mem_type(void *ptr, ucs_memory_type_t *mem_type)
     return XCCL_OK;
 }
 
+/* The last launch the calling thread put on the component's own dispatch queue
+ * without waiting for it.  Launches of that queue and of the thread's HIP
+ * stream are not ordered against each other by the device, so the thread's
+ * next launch on the stream waits for this one on the host first (rare: a
+ * small stream-ordered reduction followed by a large one). */
+static _Thread_local struct {
+    volatile uint32_t *flag;
+    int                words;
+    uint32_t           expect;
+    unsigned           generation;
+} mc_last_direct;
+
+/* bumped by close(): completion words recorded before it are gone */
+static atomic_uint mc_generation;
+
+static void mc_rocm_wait_last_direct(void)
+{
+    unsigned polls = 0;
+    int      i;
+
+    if (mc_last_direct.flag == NULL) {
+        return;
+    }
+    if (mc_last_direct.generation != atomic_load(&mc_generation)) {
+        mc_last_direct.flag = NULL;
+        return;
+    }
+    for (i = 0; i < mc_last_direct.words; i++) {
+        /* sequence numbers of a word only grow: at or past ours means ours is done */
+        while ((int32_t)(__atomic_load_n(&mc_last_direct.flag[i], __ATOMIC_ACQUIRE) - mc_last_direct.expect) < 0) {
+            if ((++polls & 0xffffu) == 0 && xccl_rocm_direct_queue_failed()) {
+                break;
+            }
+            MC_CPU_RELAX();
+        }
+    }
+    mc_last_direct.flag = NULL;
+}
+
+static int mc_rocm_stream_idle(mc_rocm_device_t *d, int slot)
+{
+    return atomic_load_explicit(&d->stream_issued[slot], memory_order_acquire) ==
+           atomic_load_explicit(&d->stream_synced[slot], memory_order_acquire);
+}
+
+/* A launch on a reduction stream has been seen complete: so have all before it. */
+static void mc_rocm_note_complete(mc_rocm_event_t *ev)
+{
+    unsigned seen;
+
+    if (ev->direct || ev->slot < 0 || ev->dev == NULL) {
+        return;
+    }
+    seen = atomic_load_explicit(&ev->dev->stream_synced[ev->slot], memory_order_relaxed);
+    while ((int)(ev->stream_seq - seen) > 0 &&
+           !atomic_compare_exchange_weak(&ev->dev->stream_synced[ev->slot], &seen, ev->stream_seq)) {
+    }
+}
+
 /* Whether the flagged launch an event stands for has completed. */
 static int mc_rocm_flag_done(const mc_rocm_event_t *ev)
 {
@@ -500,6 +564,7 @@ static xccl_status_t mc_rocm_flag_poll(mc_rocm_event_t *ev, int block)
 
     for (;;) {
         if (mc_rocm_flag_done(ev)) {
+            mc_rocm_note_complete(ev);
             return XCCL_OK;
         }
         if ((++ev->polls & 0xffffu) == 0 && ev->direct) {
@@ -537,7 +602,8 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
     mc_rocm_event_t  *ev = NULL;
     hipStream_t       hs;
     xccl_status_t     st;
-    int               flagged = 0;
+    int               flagged = 0, slot;
+    unsigned          stream_seq = 0;
 
     st = xccl_rocm_reduce_supported(dtype, op);
     if (st != XCCL_OK) {
@@ -567,29 +633,46 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
         }
     }
 
-    if (want_sync && stream == NULL && ev != NULL && mc_graph_max_bytes == 0 &&
-        atomic_load_explicit(&d->unsynced[mc_rocm_thread_slot()], memory_order_acquire) == 0) {
-        /* nothing of this thread's stream to stay behind, and the caller waits
-         * here: the launch needs no stream at all */
+    slot = stream == NULL ? mc_rocm_thread_slot() : -1;
+    if (slot >= 0 && ev != NULL && mc_graph_max_bytes == 0 && mc_rocm_stream_idle(d, slot)) {
+        /* The launch will tell its own completion, and this slot's stream holds
+         * nothing to stay behind: it needs no stream at all.  The component's
+         * own queue runs this slot's launches in order. */
         st = xccl_rocm_reduce_multi_direct(sbuf1, sbuf2, rbuf, count, size,
-                                           stride, dtype, op, mc_rocm_thread_slot(),
+                                           stride, dtype, op, slot,
                                            ev->dev_count, ev->dev_flag,
                                            MC_FLAG_STRIDE, ev->expect + 1,
                                            &flagged);
-        if (st == XCCL_OK && flagged) {
-            ev->stream  = hs;
-            ev->flagged = flagged;
-            ev->direct  = 1;
-            ev->polls   = 0;
-            ev->expect++;
-            st = mc_rocm_flag_poll(ev, 1);
-            atomic_store(&ev->is_free, MC_SLOT_FREE);
-            return st;
-        }
         if (st != XCCL_OK) {
             atomic_store(&ev->is_free, MC_SLOT_FREE);
             return st;
         }
+        if (flagged) {
+            ev->stream  = hs;
+            ev->flagged = flagged;
+            ev->direct  = 1;
+            ev->slot    = -1;
+            ev->polls   = 0;
+            ev->expect++;
+            if (want_sync) {
+                st = mc_rocm_flag_poll(ev, 1);
+            } else {
+                mc_last_direct.flag       = ev->flag;
+                mc_last_direct.words      = flagged;
+                mc_last_direct.expect     = ev->expect;
+                mc_last_direct.generation = atomic_load(&mc_generation);
+            }
+            if (event != NULL && st == XCCL_OK) {
+                ev->super.mem_type = UCS_MEMORY_TYPE_ROCM;
+                *event             = &ev->super;
+            } else {
+                atomic_store(&ev->is_free, MC_SLOT_FREE);
+            }
+            return st;
+        }
+    }
+    if (slot >= 0) {
+        mc_rocm_wait_last_direct();
     }
     if (want_sync && size * xccl_dt_size(dtype) <= mc_graph_max_bytes) {
         st = xccl_rocm_reduce_multi_graph(sbuf1, sbuf2, rbuf, count, size,
@@ -610,14 +693,17 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
         }
         return st;
     }
-    if (stream == NULL && !want_sync) {
-        atomic_store_explicit(&d->unsynced[mc_rocm_thread_slot()], 1, memory_order_release);
+    if (slot >= 0) {
+        stream_seq = atomic_fetch_add_explicit(&d->stream_issued[slot], 1, memory_order_acq_rel) + 1;
     }
     if (ev != NULL) {
-        ev->stream  = hs;
-        ev->flagged = flagged;
-        ev->direct  = 0;
-        ev->polls   = 0;
+        ev->stream     = hs;
+        ev->flagged    = flagged;
+        ev->direct     = 0;
+        ev->slot       = slot;
+        ev->stream_seq = stream_seq;
+        ev->dev        = d;
+        ev->polls      = 0;
         if (flagged) {
             ev->expect++;
         } else if (event != NULL && hipEventRecord(ev->hip_event, hs) != hipSuccess) {
@@ -630,10 +716,11 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
             st = mc_rocm_flag_poll(ev, 1);
         } else if (hipStreamSynchronize(hs) != hipSuccess) {
             st = XCCL_ERR_NO_MESSAGE;
-        }
-        if (stream == NULL && st == XCCL_OK) {
-            /* stream order: everything this slot's stream held before is complete as well */
-            atomic_store_explicit(&d->unsynced[mc_rocm_thread_slot()], 0, memory_order_release);
+        } else if (ev != NULL) {
+            mc_rocm_note_complete(ev);
+        } else if (slot >= 0) {
+            mc_rocm_event_t none = {.direct = 0, .slot = slot, .stream_seq = stream_seq, .dev = d};
+            mc_rocm_note_complete(&none);
         }
     }
     if (ev != NULL) {
@@ -720,6 +807,7 @@ static xccl_status_t mc_rocm_event_record(xccl_stream_t *stream,
     }
     ev->flagged = 0;
     ev->direct  = 0;
+    ev->slot    = -1;
     ev->stream  = hs;
     e = hipEventRecord(ev->hip_event, hs);
     if (e != hipSuccess) {
@@ -748,6 +836,7 @@ static xccl_status_t mc_rocm_event_query(xccl_mc_event_t *event)
     }
     e = hipEventQuery(mc_rocm_event_of(event)->hip_event);
     if (e == hipSuccess) {
+        mc_rocm_note_complete(mc_rocm_event_of(event));
         return XCCL_OK;
     }
     if (e == hipErrorNotReady) {
@@ -765,6 +854,7 @@ static xccl_status_t mc_rocm_event_wait(xccl_mc_event_t *event)
         return mc_rocm_flag_poll(mc_rocm_event_of(event), 1);
     }
     MC_HIP(hipEventSynchronize(mc_rocm_event_of(event)->hip_event));
+    mc_rocm_note_complete(mc_rocm_event_of(event));
     return XCCL_OK;
 }
 
@@ -891,6 +981,7 @@ static void mc_rocm_close(void)
         return;
     }
     mc_pool_trim(-1);
+    atomic_fetch_add(&mc_generation, 1);
     pthread_mutex_lock(&mc_init_lock);
     for (dev = 0; dev < MC_MAX_DEVICES; dev++) {
         d = &mc_devices[dev];
