@@ -39,10 +39,12 @@ extern "C" {
 
 /* Looks up what the launchers need to know about the CURRENT device (its
  * compute-unit count, the address of the library's static counter array on
- * it) so that later calls on that device make no runtime query.  Optional:
- * the launchers do the same on their first call on a device; a caller that
- * will launch from inside a stream capture calls this once outside it.  The
- * component calls it when it sets a device up. */
+ * it) so that later calls on that device make no runtime query, and sets up
+ * the dispatch queues of xccl_rocm_reduce_multi_direct there (loads the
+ * kernels' code objects, creates the queues: milliseconds, and allocations).
+ * Optional: the launchers do the same on their first call on a device; a
+ * caller that will launch from inside a stream capture calls this once
+ * outside it.  The component calls it when it sets a device up. */
 xccl_status_t xccl_rocm_prepare_device(void);
 
 /* XCCL_OK if a kernel exists for (dtype, op), XCCL_ERR_UNSUPPORTED if not.

@@ -783,17 +783,17 @@ bool direct_queue(DirectDevice &dd, int slot, DirectQueue **out)
     return true;
 }
 
-// Puts `plan` on queue `slot` of the current device.  Anything but XCCL_OK:
-// nothing was enqueued and the caller launches on a HIP stream instead.
-xccl_status_t direct_launch(int slot, const Plan &plan)
+// The current device's queues and code, set up on first use; NULL when the
+// path is off or could not be set up.
+DirectDevice *direct_device()
 {
-    if (!direct_enabled() || g_direct_failed.load(std::memory_order_acquire) != 0 || slot < 0 || slot >= kDirectQueues) {
-        return XCCL_ERR_NO_RESOURCE;
+    if (!direct_enabled() || g_direct_failed.load(std::memory_order_acquire) != 0) {
+        return nullptr;
     }
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         (void)hipGetLastError();
-        return XCCL_ERR_NO_RESOURCE;
+        return nullptr;
     }
     DirectDevice &dd    = g_direct[dev];
     int           state = dd.state.load(std::memory_order_acquire);
@@ -805,9 +805,21 @@ xccl_status_t direct_launch(int slot, const Plan &plan)
             dd.state.store(state, std::memory_order_release);
         }
     }
-    if (state != 1) {
+    return state == 1 ? &dd : nullptr;
+}
+
+// Puts `plan` on queue `slot` of the current device.  Anything but XCCL_OK:
+// nothing was enqueued and the caller launches on a HIP stream instead.
+xccl_status_t direct_launch(int slot, const Plan &plan)
+{
+    if (slot < 0 || slot >= kDirectQueues) {
         return XCCL_ERR_NO_RESOURCE;
     }
+    DirectDevice *found = direct_device();
+    if (found == nullptr) {
+        return XCCL_ERR_NO_RESOURCE;
+    }
+    DirectDevice &dd = *found;
     DirectKernel k;
     DirectQueue *dq = nullptr;
     if (!direct_kernel(dd, plan.fn, &k) || !direct_queue(dd, slot, &dq)) {
@@ -892,7 +904,22 @@ xccl_status_t xccl_rocm_prepare_device(void)
     int           cus = 0;
     uint32_t     *p   = nullptr;
     xccl_status_t st  = cu_count(&cus);
-    return st != XCCL_OK ? st : static_scratch(&p);
+    if (st == XCCL_OK) {
+        st = static_scratch(&p);
+    }
+    if (st == XCCL_OK) {
+        // the component's own dispatch queues: loading the code and creating the queues takes milliseconds,
+        // which belong here and not into the first small reduction; failure leaves the stream path
+        DirectDevice *dd = direct_device();
+        for (int slot = 0; dd != nullptr && slot < kDirectQueues; ++slot) {
+            DirectQueue *dq = nullptr;
+            if (!direct_queue(*dd, slot, &dq)) {
+                dd->state.store(-1, std::memory_order_release);
+                break;
+            }
+        }
+    }
+    return st;
 }
 
 xccl_status_t xccl_rocm_reduce_supported(xccl_dt_t dtype, xccl_op_t op)
