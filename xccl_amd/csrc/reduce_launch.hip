@@ -577,12 +577,14 @@ int arm_completion(Plan &plan, uint32_t *dev_count, uint32_t *dev_flag, uint32_t
 // fences, which is what a kernel launched on a HIP stream gets; the result
 // stores are write-through and waited for by the kernel itself.
 //   Two queues per device, for the first two of the component's four thread
-// slots; threads of the other slots keep to their HIP streams.  Measured,
-// blocking call, 4 sources x 1 KiB, p50 / p99 in us: one thread 5.6 / 5.9; two
-// threads on a queue each 5.6 / 7.8; four threads on a queue each 9.4 / 30
-// (queues beyond what the hardware keeps mapped get time-sliced); four threads
-// sharing one queue 13.3 / 13.6 (the packet processor takes ~3 us per packet
-// of a queue, fences included, one after the other).
+// slots, each created when a thread of the slot first calls, behind that
+// slot's HIP stream; threads of the other slots keep to their HIP streams.
+// Measured, blocking call, 4 sources x 1 KiB, p50 / p99 in us: one thread 5.4 /
+// 5.7; two threads on a queue each 5.6-6.0 / 6.8-8.4; four threads on a queue
+// each 9.5 / 30 (twice, on different boxes), two of them on HIP streams instead
+// 7.4 / 11.2, all four on HIP streams 7.2 / 13.4; four threads sharing one queue
+// 13.3 / 13.6 (the packet processor takes ~3 us per packet of a queue, fences
+// included, one after the other).
 extern "C" {
 extern const unsigned char *const xccl_rocm_kernel_image_begin[5];
 extern const unsigned char *const xccl_rocm_kernel_image_end[5];
@@ -908,15 +910,15 @@ xccl_status_t xccl_rocm_prepare_device(void)
         st = static_scratch(&p);
     }
     if (st == XCCL_OK) {
-        // the component's own dispatch queues: loading the code and creating the queues takes milliseconds,
-        // which belong here and not into the first small reduction; failure leaves the stream path
+        // the component's own dispatch queue: loading the code and creating a queue takes milliseconds, which
+        // belong here and not into the first small reduction; failure leaves the stream path.  Only the first
+        // calling thread's queue: the others are created when a thread of their slot first calls.  (The
+        // device serves the queue created last fastest: an empty kernel's completion word is seen 4.6 us
+        // after the doorbell on the newest of up to 12 open queues, 4.8-5.5 us on the older ones.)
         DirectDevice *dd = direct_device();
-        for (int slot = 0; dd != nullptr && slot < kDirectQueues; ++slot) {
-            DirectQueue *dq = nullptr;
-            if (!direct_queue(*dd, slot, &dq)) {
-                dd->state.store(-1, std::memory_order_release);
-                break;
-            }
+        DirectQueue  *dq = nullptr;
+        if (dd != nullptr && !direct_queue(*dd, 0, &dq)) {
+            dd->state.store(-1, std::memory_order_release);
         }
     }
     return st;
