@@ -42,6 +42,10 @@ std::atomic<int> g_blocks_per_cu{-1}; // -1: not read from the environment yet
 std::atomic<int> g_resident{0};
 std::atomic<int> g_tail_flag{1};
 std::atomic<unsigned> g_shape_epoch{0}; // bumped when a launch-shape knob changes
+// the same bound for launches on the component's own dispatch queue, where the alternative to counting is the
+// stream path as a whole (blocking call, us, counting on the own queue / queued kernel on the stream: 3072
+// workgroups 7.8 / 8.8-9.3, 4096: 8.2 / 8.9-9.4, 6144: 9.2 / 9.2-9.4, 8192: 10.0 / 9.6-9.8)
+std::atomic<unsigned> g_direct_counted_grid{6144};
 std::atomic<unsigned> g_max_counted_grid{2048}; // measured (blocking call, us, counting / queued kernel): 512 workgroups 8.0 / 9.2, 2048: 8.6-9.7 / 9.4-9.5, 8192: 10.4 / 10.0
 // Launches of at most this many workgroups (and at least 4 sources; up to 3 the
 // walk has every load in flight anyway) use the burst kernel: all loads of a
@@ -78,6 +82,7 @@ void read_env_once()
     const char *mcg = getenv("XCCL_MC_ROCM_MAX_COUNTED_GRID");
     if (mcg != nullptr && atoi(mcg) >= 0 && (unsigned)atoi(mcg) <= kMaxFlaggedGrid) {
         g_max_counted_grid.store((unsigned)atoi(mcg), std::memory_order_release);
+        g_direct_counted_grid.store((unsigned)atoi(mcg), std::memory_order_release);
     }
     int         v   = bpc ? atoi(bpc) : 0;
     g_resident.store(res && atoi(res) > 0 ? atoi(res) : 0, std::memory_order_release);
@@ -959,7 +964,7 @@ xccl_status_t xccl_rocm_reduce_multi_direct(void *sbuf1, void *sbuf2, void *rbuf
     if (st != XCCL_OK || nothing) {
         return st;
     }
-    if (plan.grid > g_max_counted_grid.load(std::memory_order_relaxed) || plan.grid > kMaxFlaggedGrid) {
+    if (plan.grid > g_direct_counted_grid.load(std::memory_order_relaxed) || plan.grid > kMaxFlaggedGrid) {
         return XCCL_OK; // completes through the stream: not for this queue
     }
     const int words = arm_completion(plan, dev_count, dev_flag, flag_words, seq);
