@@ -539,6 +539,34 @@ def test_blocking_calls_take_the_components_own_queue(rocm, oracle):
             assert time.time() - t0 < 20.0
         assert rocm.xccl_mc_event_free(ev_small) == Status.OK and rocm.xccl_mc_event_free(ev_large) == Status.OK
         assert blocking(small, "own queue: the large launch has been seen complete") == 1
+        # 48 stream-ordered calls in place, none waited for until the end: the queue runs them in order
+        chain = Case(Dt.INT32, 3000, 1, alias="s1")
+        try:
+            chain.fill_random(oracle, 44, Op.SUM)
+            chain.upload()
+            c1, c2, cr = chain.ptrs()
+            assert cr == c1
+            assert blocking(small, "the stream is idle as far as the component has seen") == 1
+            before = lib.xccl_rocm_direct_launch_count()
+            evs = []
+            for rep in range(48):
+                st, e = rocm.xccl_mem_component_reduce_multi_nb(c1, c2, cr, 1, chain.size, chain.stride, Dt.INT32, Op.SUM,
+                                                                MemType.ROCM, None)
+                assert st == Status.OK and e is not None
+                evs.append(e)
+            assert lib.xccl_rocm_direct_launch_count() - before == 48
+            t0 = time.time()
+            while rocm.xccl_mc_event_query(evs[-1]) == Status.INPROGRESS:
+                assert time.time() - t0 < 20.0
+            for e in evs:
+                assert rocm.xccl_mc_event_query(e) == Status.OK
+                assert rocm.xccl_mc_event_free(e) == Status.OK
+            a = chain.host[chain.o1: chain.o1 + chain.vbytes].view(np.int32).astype(np.int64)
+            b = chain.host[chain.o2: chain.o2 + chain.vbytes].view(np.int32).astype(np.int64)
+            want = ((a + 48 * b) & 0xffffffff).astype(np.uint32).view(np.int32)
+            assert chain.result().view(np.int32).tolist() == want.tolist()
+        finally:
+            chain.close()
         # 2000 in a row: kernel-argument slots and packets are reused many times over
         p1, p2, pr = small.ptrs()
         before = lib.xccl_rocm_direct_launch_count()

@@ -598,6 +598,10 @@ extern const unsigned char *const xccl_rocm_kernel_image_end[5];
 constexpr int      kDirectQueues  = 2;
 constexpr uint32_t kDirectPackets = 256; // queue size; a blocking caller has one launch in flight
 constexpr size_t   kKernargSlot   = 128; // >= sizeof(ReduceArgs), one cache line pair per packet
+// Twice as many argument slots as packets: a packet is written once the queue has *consumed* the one 256
+// before it, which may still be running; with 512 slots an argument block is rewritten only after the packet
+// 256 behind its last user has been consumed, and the barrier bit makes that wait for everything before it.
+constexpr uint32_t kKernargSlots  = 2 * kDirectPackets;
 static_assert(sizeof(ReduceArgs) <= kKernargSlot, "kernel argument slot");
 
 struct DirectKernel {
@@ -607,7 +611,7 @@ struct DirectKernel {
 
 struct DirectQueue {
     hsa_queue_t *q       = nullptr;
-    char        *kernarg = nullptr; // kDirectPackets slots, pinned host memory
+    char        *kernarg = nullptr; // kKernargSlots slots, pinned host memory
 };
 
 struct DirectDevice {
@@ -765,11 +769,11 @@ bool direct_queue(DirectDevice &dd, int slot, DirectQueue **out)
         std::lock_guard<std::mutex> guard(dd.lock);
         if (dq.q == nullptr) {
             char *ring = nullptr;
-            if (hipHostMalloc((void **)&ring, kDirectPackets * kKernargSlot, hipHostMallocDefault) != hipSuccess) {
+            if (hipHostMalloc((void **)&ring, kKernargSlots * kKernargSlot, hipHostMallocDefault) != hipSuccess) {
                 (void)hipGetLastError();
                 return false;
             }
-            memset(ring, 0, kDirectPackets * kKernargSlot);
+            memset(ring, 0, kKernargSlots * kKernargSlot);
             hsa_queue_t *q = nullptr;
             hsa_status_t st = hsa_queue_create(dd.agent, kDirectPackets, HSA_QUEUE_TYPE_MULTI, on_queue_error, nullptr,
                                                UINT32_MAX, UINT32_MAX, &q);
@@ -840,9 +844,12 @@ xccl_status_t direct_launch(int slot, const Plan &plan)
     hsa_queue_t   *q   = dq->q;
     const uint64_t idx = hsa_queue_add_write_index_scacq_screl(q, 1);
     while (idx - hsa_queue_load_read_index_scacquire(q) >= q->size) {
-        // queue full: more than kDirectPackets launches of blocking callers in flight; wait for the oldest
+        // queue full: kDirectPackets launches waiting to start; wait for the oldest
+        if (g_direct_failed.load(std::memory_order_acquire) != 0) {
+            return XCCL_ERR_NO_RESOURCE; // the queue is dead; the reserved packet stays invalid
+        }
     }
-    char *args = dq->kernarg + (idx & (kDirectPackets - 1)) * kKernargSlot;
+    char *args = dq->kernarg + (idx & (kKernargSlots - 1)) * kKernargSlot;
     memcpy(args, &plan.args, sizeof(ReduceArgs));
 
     hsa_kernel_dispatch_packet_t *p = static_cast<hsa_kernel_dispatch_packet_t *>(q->base_address) + (idx & (q->size - 1));
