@@ -623,12 +623,14 @@ def test_many_events_in_flight_any_wait_order(rocm, oracle):
 
 def test_blocking_calls_from_several_threads(rocm, oracle):
     """test/test_mt.c runs 4 threads of collectives; the component's pools and
-    lazy initialisation must hold up: 4 threads x 200 blocking reductions on
-    private buffers, every result checked."""
+    lazy initialisation must hold up: 8 threads x 300 blocking reductions on
+    private buffers, every result checked.  Eight threads share the four
+    thread slots in pairs, so each of the component's own dispatch queues has
+    two producers at once."""
     import threading
     dt, op, size = Dt.INT32, Op.SUM, 4096
     cases = []
-    for t in range(4):
+    for t in range(8):
         c = Case(dt, size + t, 3)
         c.fill_random(oracle, 70 + t)
         c.upload()
@@ -639,12 +641,12 @@ def test_blocking_calls_from_several_threads(rocm, oracle):
         try:
             p1, p2, pr = c.ptrs()
             want, _ = c.expect(oracle, op)
-            for rep in range(200):
+            for rep in range(300):
                 st = rocm.xccl_mem_component_reduce_multi(p1, p2, pr, 3, c.size, c.stride, dt, op, MemType.ROCM)
                 if st != Status.OK:
                     errors.append(st)
                     return
-                if rep % 40 == 0:
+                if rep % 60 == 0:
                     assert_same(c.result(), want, dt, op, "thread size %d rep %d" % (c.size, rep))
         except Exception as e:  # noqa: BLE001
             errors.append(e)
