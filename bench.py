@@ -153,7 +153,14 @@ def latency_sweep(mc, hip, iters, quick):
     """Config 5: FLOAT32 SUM, 2/4/8 sources, 4 B .. 32 KiB per vector, `iters` back-to-back calls per cell."""
     from xccl_amd.types import Dt, Op, Status
     sizes_b = [4, 1024, 32768] if quick else [4 << k for k in range(14)]
-    res = {"iterations_per_cell": iters, "bytes_per_vector": sizes_b}
+    res = {"iterations_per_cell": iters, "bytes_per_vector": sizes_b,
+           "modes": {"sync": "blocking vtable entry (launches on the component's own dispatch queue)",
+                     "event": "reduce_multi_nb + event_query until done (own dispatch queue)",
+                     "issue": "reduce_multi_nb with an event: host time of the call alone",
+                     "sync_on_hip_stream": "blocking vtable entry with the own queue switched off: hipLaunchKernel on "
+                                           "the component's stream, completion word",
+                     "stream": "reduce_multi_nb without an event + hipStreamSynchronize",
+                     "graph": "cached one-node hipGraph launch + hipStreamSynchronize"}}
     maxb = 32768
     buf = hip.DeviceBuffer(10 * maxb)
     for j in range(9):
