@@ -780,6 +780,46 @@ def test_first_use_of_a_device_inside_a_capture_is_refused():
     assert "inside a stream capture" in out.stderr
 
 
+def test_component_works_again_after_close():
+    """close() releases a device's streams, events, dispatch queues and the
+    code loaded for them; the next call sets everything up again.  A fresh
+    process: reductions on the own queue and on the stream, close (through the
+    dispatcher's free_cache), the same reductions once more."""
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import sys\n"
+        "sys.path.insert(0, %r)\n"
+        "import numpy as np\n"
+        "from xccl_amd import hip, mc\n"
+        "from xccl_amd.types import Dt, MemType, Op, Status\n"
+        "hip.set_device(0)\n"
+        "assert mc.xccl_mem_component_init() == Status.OK\n"
+        "lib = mc.component_lib()\n"
+        "n = 1 << 22\n"
+        "buf = hip.DeviceBuffer(3 * n * 4)\n"
+        "buf.upload(np.arange(2 * n, dtype=np.float32))\n"
+        "want = np.arange(n, dtype=np.float32) + np.arange(n, 2 * n, dtype=np.float32)\n"
+        "def run(count):\n"
+        "    hip.memset(buf.ptr + 2 * n * 4, 0, count * 4)\n"
+        "    hip.device_synchronize()\n"
+        "    before = lib.xccl_rocm_direct_launch_count()\n"
+        "    st = mc.xccl_mem_component_reduce_multi(buf.ptr, buf.ptr + n * 4, buf.ptr + 2 * n * 4, 1, count, n * 4,\n"
+        "                                            Dt.FLOAT32, Op.SUM, MemType.ROCM)\n"
+        "    got = buf.download(np.float32, count, 2 * n * 4)\n"
+        "    return int(st), int(lib.xccl_rocm_direct_launch_count() - before), bool((got == want[:count]).all())\n"
+        "a = [run(1000), run(1000), run(n)]\n"
+        "mc.xccl_mem_component_free_cache()\n"
+        "b = [run(1000), run(1000), run(n)]\n"
+        "print('before', a, 'after', b)\n"
+    ) % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    expect = "[(0, 1, True), (0, 1, True), (0, 0, True)]"
+    assert "before %s after %s" % (expect, expect) in out.stdout, out.stdout + out.stderr
+
+
 def test_graph_launch_with_completion_word(rocm, oracle):
     """xccl_rocm_reduce_multi_graph_flagged: the one-node graph launch that
     carries the kernel-written completion word (its sequence number is a kernel

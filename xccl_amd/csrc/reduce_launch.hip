@@ -616,6 +616,7 @@ struct DirectQueue {
 
 struct DirectDevice {
     std::atomic<int>                              state{0}; // 0 untried, 1 usable, -1 unavailable
+    std::atomic<unsigned>                         generation{0}; // bumped when the executable is destroyed
     std::mutex                                    lock;
     hsa_agent_t                                   agent{};
     hsa_executable_t                              exe{};
@@ -727,7 +728,9 @@ bool direct_kernel(DirectDevice &dd, const void *fn, DirectKernel *out)
     thread_local const void  *last_fn = nullptr;
     thread_local DirectKernel last;
     thread_local const DirectDevice *last_dd = nullptr;
-    if (fn == last_fn && last_dd == &dd) {
+    thread_local unsigned            last_gen = 0;
+    const unsigned                   gen      = dd.generation.load(std::memory_order_acquire);
+    if (fn == last_fn && last_dd == &dd && last_gen == gen) {
         *out = last;
         return true;
     }
@@ -755,10 +758,11 @@ bool direct_kernel(DirectDevice &dd, const void *fn, DirectKernel *out)
         }
         it = dd.kernels.emplace(fn, k).first;
     }
-    *out    = it->second;
-    last    = it->second;
-    last_fn = fn;
-    last_dd = &dd;
+    *out     = it->second;
+    last     = it->second;
+    last_fn  = fn;
+    last_dd  = &dd;
+    last_gen = gen;
     return true;
 }
 
@@ -894,6 +898,7 @@ void direct_destroy(DirectDevice &dd)
         }
     }
     dd.kernels.clear();
+    dd.generation.fetch_add(1, std::memory_order_release); // kernel descriptors cached by the threads are stale now
     if (dd.exe.handle != 0) {
         (void)hsa_executable_destroy(dd.exe);
         dd.exe.handle = 0;
