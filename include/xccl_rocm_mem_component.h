@@ -164,8 +164,9 @@ typedef struct xccl_rocm_mem_component {
 
 /* Defined by xccl_rocm_mem_component.so; xccl_cuda_mem_component is an alias
  * of the same object.  xccl_rocm_mem_component_ext points at it: a loader
- * that wants the extension looks THAT symbol up, so it never has to read
- * behind the vtable of a component that may not have one. */
+ * that wants the extension looks THAT symbol up
+ * (xccl_<memory type name>_mem_component_ext), so it never has to read behind
+ * the vtable of a component that may not have one. */
 extern xccl_rocm_mem_component_t        xccl_rocm_mem_component;
 extern xccl_rocm_mem_component_t *const xccl_rocm_mem_component_ext;
 
@@ -178,7 +179,8 @@ extern xccl_rocm_mem_component_t *const xccl_rocm_mem_component_ext;
  * every non-host memory type (names host, cuda, cuda-managed, rocm,
  * rocm-managed).  The data symbol is looked up as `xccl_<name>_mem_component`
  * ('-' -> '_') first and as `xccl_cuda_mem_component` second; a file that
- * exports neither is skipped (the reference dereferences NULL there).
+ * exports neither is skipped (the reference dereferences NULL there).  The
+ * extension is taken from `xccl_<name>_mem_component_ext` if the file has it.
  * Cache size comes from XCCL_MEM_COMPONENT_CACHE_SIZE (default 4096,
  * reference src/core/xccl_global_opts.c:3-37). */
 xccl_status_t xccl_mem_component_init(const char *components_path);
@@ -204,8 +206,22 @@ xccl_status_t xccl_mem_component_reduce_multi(void *sbuf1, void *sbuf2,
                                               xccl_dt_t dtype, xccl_op_t op,
                                               ucs_memory_type_t mem_type);
 
-/* Stream-ordered forms (extension; XCCL_ERR_NOT_IMPLEMENTED when the loaded
- * component has no extension). */
+/* Stream-ordered forms: the two entries integration/xccl-rocm.patch adds to
+ * the reference's src/utils/mem_component.{h,c}, with the same arguments and
+ * the same rule (an in-tree build, -DXCCL_MC_ROCM_IN_TREE, sees both
+ * declarations and fails on any difference).  What the patched call sites of
+ * the UCX team library call (allreduce_knomial.c:74-80,129-135,
+ * allreduce_sra.c:212-218,281-284, reduce_knomial.c:79-85,
+ * reduce_linear.c:28-34), always with stream == NULL.
+ *   stream == NULL : the component's queue of the calling thread
+ *   event  != NULL : *event is NULL when the reduction is complete on return,
+ *                    else an event for xccl_mc_event_query / _free
+ * Fallbacks, in this order: host memory or no component -> whatever the
+ * blocking entry above returns; component without the extension -> the
+ * blocking entry if stream == NULL, else XCCL_ERR_NOT_IMPLEMENTED; empty
+ * reduction -> XCCL_OK; the component's event pool is empty
+ * (XCCL_ERR_NO_RESOURCE, nothing enqueued) -> the blocking entry if
+ * stream == NULL, else that error. */
 xccl_status_t xccl_mem_component_reduce_nb(void *sbuf1, void *sbuf2,
                                            void *target, size_t count,
                                            xccl_dt_t dtype, xccl_op_t op,

@@ -168,8 +168,10 @@ def test_dt_size():
 @pytest.fixture(scope="module")
 def fake(tmp_path_factory):
     """Builds tests/fake_component.c as xccl_cuda_mem_component.so (exports the
-    hard-coded name) and xccl_cuda-managed_mem_component.so (exports its own
-    name only), and loads them through xccl_mem_component_init."""
+    hard-coded name, plain reference vtable) and
+    xccl_cuda-managed_mem_component.so (exports its own name only, and the
+    stream-ordered extension under xccl_cuda_managed_mem_component_ext), and
+    loads them through xccl_mem_component_init."""
     d = tmp_path_factory.mktemp("plugins")
     src = os.path.join(ROOT, "tests", "fake_component.c")
     libs = {}
@@ -177,8 +179,9 @@ def fake(tmp_path_factory):
                            ("xccl_cuda-managed_mem_component.so", "xccl_cuda_managed_mem_component",
                             MemType.CUDA_MANAGED)):
         out = os.path.join(str(d), fname)
-        subprocess.run(["gcc", "-shared", "-fPIC", "-O1", "-I", INC, "-DFAKE_SYMBOL=" + sym,
-                        "-DFAKE_MEMTYPE=%d" % int(mt), "-o", out, src], check=True)
+        ext = ["-DFAKE_EXT_SYMBOL=%s_ext" % sym] if mt == MemType.CUDA_MANAGED else []
+        subprocess.run(["gcc", "-shared", "-fPIC", "-O1", "-Wall", "-Werror", "-I", INC, "-DFAKE_SYMBOL=" + sym,
+                        "-DFAKE_MEMTYPE=%d" % int(mt), "-o", out, src] + ext, check=True)
         libs[mt] = ctypes.CDLL(out)
     # a file that exports neither name must be skipped, not dereferenced
     bad = os.path.join(str(d), "xccl_rocm-managed_mem_component.so")
@@ -274,11 +277,67 @@ def test_reduce_forwarding_and_error_codes(fake):
     assert mc.xccl_mem_component_reduce(1, 2, 3, 4, Dt.INT32, Op.SUM, MemType.HOST) == Status.ERR_UNSUPPORTED
     assert mc.xccl_mem_component_reduce_multi(1, 2, 3, 1, 4, 16, Dt.INT32, Op.SUM,
                                               MemType.HOST) == Status.ERR_UNSUPPORTED
-    # a component without the stream-ordered extension
-    st, _ = mc.xccl_mem_component_reduce_multi_nb(1, 2, 3, 1, 4, 16, Dt.INT32, Op.SUM, MemType.CUDA)
-    assert st == Status.ERR_NOT_IMPLEMENTED
-    st, _ = mc.xccl_mem_component_reduce_nb(1, 2, 3, 4, Dt.INT32, Op.SUM, MemType.ROCM_MANAGED)
-    assert st == Status.ERR_UNSUPPORTED
+
+
+def test_stream_ordered_entries_and_their_fallback_rule(fake):
+    """The *_nb dispatcher entries (the ones integration/xccl-rocm.patch adds to
+    reference src/utils/mem_component.c): one fallback rule, followed here by
+    every branch."""
+    plain, ext = fake[MemType.CUDA], fake[MemType.CUDA_MANAGED]
+    s = mc.Stream(0x1234, StreamType.CUDA)
+    # a component without the extension, no stream named: the blocking entry runs, no event
+    n0 = _calls(plain)
+    st, ev = mc.xccl_mem_component_reduce_multi_nb(0x10, 0x20, 0x30, 3, 55, 220, Dt.FLOAT32, Op.MAX, MemType.CUDA)
+    assert (st, ev) == (Status.OK, None) and _calls(plain)[5] == n0[5] + 1
+    assert list((ctypes.c_size_t * 8).in_dll(plain, "fake_last_args")) == [0x10, 0x20, 0x30, 3, 55, 220,
+                                                                           int(Dt.FLOAT32), int(Op.MAX)]
+    st, ev = mc.xccl_mem_component_reduce_nb(0x10, 0x20, 0x30, 77, Dt.INT32, Op.SUM, MemType.CUDA)
+    assert (st, ev) == (Status.OK, None) and _calls(plain)[4] == n0[4] + 1
+    # ... a stream named: nothing can keep that order
+    st, ev = mc.xccl_mem_component_reduce_multi_nb(0x10, 0x20, 0x30, 3, 55, 220, Dt.FLOAT32, Op.MAX, MemType.CUDA, s)
+    assert (st, ev) == (Status.ERR_NOT_IMPLEMENTED, None) and _calls(plain)[5] == n0[5] + 1
+    # no component / host memory: what the blocking dispatcher entry says
+    st, ev = mc.xccl_mem_component_reduce_nb(1, 2, 3, 4, Dt.INT32, Op.SUM, MemType.ROCM_MANAGED)
+    assert (st, ev) == (Status.ERR_UNSUPPORTED, None)
+    st, ev = mc.xccl_mem_component_reduce_multi_nb(1, 2, 3, 1, 4, 16, Dt.INT32, Op.SUM, MemType.HOST)
+    assert (st, ev) == (Status.ERR_UNSUPPORTED, None)
+    # a component with the extension: forwarded with the stream, event stamped with the memory type
+    ext.fake_set_nb_status(int(Status.OK))
+    n0 = _calls(ext)
+    st, ev = mc.xccl_mem_component_reduce_multi_nb(0x10, 0x20, 0x30, 3, 55, 220, Dt.FLOAT32, Op.MAX,
+                                                   MemType.CUDA_MANAGED)
+    assert st == Status.OK and ctypes.c_int.from_address(ev).value == MemType.CUDA_MANAGED
+    assert _calls(ext)[14] == n0[14] + 1 and _calls(ext)[5] == n0[5]
+    assert ctypes.c_void_p.in_dll(ext, "fake_last_stream").value is None
+    st, ev = mc.xccl_mem_component_reduce_nb(0x10, 0x20, 0x30, 77, Dt.INT32, Op.SUM, MemType.CUDA_MANAGED, s)
+    assert st == Status.OK and ev and _calls(ext)[13] == n0[13] + 1
+    assert ctypes.c_void_p.in_dll(ext, "fake_last_stream").value == ctypes.addressof(s.xccl)
+    st, ev = mc.xccl_mem_component_reduce_nb(0x10, 0x20, 0x30, 77, Dt.INT32, Op.SUM, MemType.CUDA_MANAGED, s,
+                                             want_event=False)
+    assert (st, ev) == (Status.OK, None) and _calls(ext)[13] == n0[13] + 2
+    # an empty reduction: complete on return, nothing forwarded
+    st, ev = mc.xccl_mem_component_reduce_multi_nb(0x10, 0x20, 0x30, 3, 0, 220, Dt.FLOAT32, Op.MAX,
+                                                   MemType.CUDA_MANAGED)
+    assert (st, ev) == (Status.OK, None) and _calls(ext)[14] == n0[14] + 1
+    st, ev = mc.xccl_mem_component_reduce_nb(0x10, 0x20, 0x30, 0, Dt.INT32, Op.SUM, MemType.CUDA_MANAGED)
+    assert (st, ev) == (Status.OK, None) and _calls(ext)[13] == n0[13] + 2
+    # the component has no event left: without a stream the blocking entry runs instead ...
+    ext.fake_set_nb_status(int(Status.ERR_NO_RESOURCE))
+    n1 = _calls(ext)
+    st, ev = mc.xccl_mem_component_reduce_multi_nb(0x10, 0x20, 0x30, 3, 55, 220, Dt.FLOAT32, Op.MAX,
+                                                   MemType.CUDA_MANAGED)
+    assert (st, ev) == (Status.OK, None) and _calls(ext)[14] == n1[14] + 1 and _calls(ext)[5] == n1[5] + 1
+    st, ev = mc.xccl_mem_component_reduce_nb(0x10, 0x20, 0x30, 77, Dt.INT32, Op.SUM, MemType.CUDA_MANAGED)
+    assert (st, ev) == (Status.OK, None) and _calls(ext)[13] == n1[13] + 1 and _calls(ext)[4] == n1[4] + 1
+    # ... with one the caller is told
+    st, ev = mc.xccl_mem_component_reduce_multi_nb(0x10, 0x20, 0x30, 3, 55, 220, Dt.FLOAT32, Op.MAX,
+                                                   MemType.CUDA_MANAGED, s)
+    assert (st, ev) == (Status.ERR_NO_RESOURCE, None) and _calls(ext)[5] == n1[5] + 1
+    # any other failure is passed on
+    ext.fake_set_nb_status(int(Status.ERR_UNSUPPORTED))
+    st, ev = mc.xccl_mem_component_reduce_nb(0x10, 0x20, 0x30, 77, Dt.INT32, Op.SUM, MemType.CUDA_MANAGED)
+    assert (st, ev) == (Status.ERR_UNSUPPORTED, None) and _calls(ext)[4] == n1[4] + 1
+    ext.fake_set_nb_status(int(Status.OK))
 
 
 def test_stream_routed_entries(fake):

@@ -15,7 +15,9 @@
  *   - the cached buffer is claimed atomically (mem_component.c:68-82 tests and
  *     sets `used` without synchronisation although collectives may be posted
  *     from several threads);
- *   - the *_nb / event_wait entries forward to the component's extension.
+ *   - the *_nb entries are the ones integration/xccl-rocm.patch adds to the
+ *     reference's dispatcher (same arguments, same fallback rule);
+ *     xccl_mc_event_wait and xccl_mem_component_get exist only here.
  */
 #include "xccl_rocm_mem_component.h"
 
@@ -105,9 +107,12 @@ xccl_status_t xccl_mem_component_init(const char *components_path)
             continue;
         }
         {
-            /* the extension announces itself through a symbol of its own */
-            xccl_rocm_mem_component_t **ext =
-                (xccl_rocm_mem_component_t **)dlsym(handle, "xccl_rocm_mem_component_ext");
+            /* the extension announces itself through a symbol of its own,
+             * xccl_<name>_mem_component_ext, which points at the object */
+            xccl_rocm_mem_component_t **ext;
+
+            strncat(sym, "_ext", sizeof(sym) - strlen(sym) - 1);
+            ext = (xccl_rocm_mem_component_t **)dlsym(handle, sym);
             mem_extensions[mt] = (ext != NULL && *ext != NULL && &(*ext)->super == mc &&
                                   (*ext)->ext_version >= 1) ? *ext : NULL;
         }
@@ -209,36 +214,78 @@ xccl_status_t xccl_mem_component_reduce_multi(void *sbuf1, void *sbuf2, void *rb
     return mc->reduce_multi(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op);
 }
 
+/*
+ * Stream-ordered forms -- the same entries, argument for argument and rule
+ * for rule, that integration/xccl-rocm.patch adds to the reference's
+ * src/utils/mem_component.{h,c}:
+ *   - *event (if asked for) is NULL whenever the reduction is complete on
+ *     return;
+ *   - host memory or no component: the blocking dispatcher entry decides;
+ *   - a component without the extension: the blocking entry when the call
+ *     names no stream, XCCL_ERR_NOT_IMPLEMENTED when it does;
+ *   - an empty reduction is XCCL_OK;
+ *   - an empty event pool (XCCL_ERR_NO_RESOURCE from the component, nothing
+ *     enqueued): the blocking entry when the call names no stream, the error
+ *     when it does.
+ */
 xccl_status_t xccl_mem_component_reduce_nb(void *sbuf1, void *sbuf2, void *target, size_t count, xccl_dt_t dtype,
                                            xccl_op_t op, ucs_memory_type_t mt, xccl_stream_t *stream,
                                            xccl_mc_event_t **event)
 {
-    xccl_rocm_mem_component_t *ext;
+    xccl_mem_component_t      *mc  = component_of(mt);
+    xccl_rocm_mem_component_t *ext = extension_of(mt);
+    xccl_status_t              st;
 
-    if (component_of(mt) == NULL) {
-        return XCCL_ERR_UNSUPPORTED;
+    if (event != NULL) {
+        *event = NULL;
     }
-    ext = extension_of(mt);
+    if (mc == NULL || (ext == NULL && stream == NULL)) {
+        return xccl_mem_component_reduce(sbuf1, sbuf2, target, count, dtype, op, mt);
+    }
     if (ext == NULL) {
         return XCCL_ERR_NOT_IMPLEMENTED;
     }
-    return ext->reduce_nb(sbuf1, sbuf2, target, count, dtype, op, stream, event);
+    if (count == 0) {
+        return XCCL_OK;
+    }
+    st = ext->reduce_nb(sbuf1, sbuf2, target, count, dtype, op, stream, event);
+    if (st == XCCL_ERR_NO_RESOURCE && stream == NULL) {
+        return mc->reduce(sbuf1, sbuf2, target, count, dtype, op);
+    }
+    if (st == XCCL_OK && event != NULL) {
+        (*event)->mem_type = mt;
+    }
+    return st;
 }
 
 xccl_status_t xccl_mem_component_reduce_multi_nb(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
                                                  size_t stride, xccl_dt_t dtype, xccl_op_t op, ucs_memory_type_t mt,
                                                  xccl_stream_t *stream, xccl_mc_event_t **event)
 {
-    xccl_rocm_mem_component_t *ext;
+    xccl_mem_component_t      *mc  = component_of(mt);
+    xccl_rocm_mem_component_t *ext = extension_of(mt);
+    xccl_status_t              st;
 
-    if (component_of(mt) == NULL) {
-        return XCCL_ERR_UNSUPPORTED;
+    if (event != NULL) {
+        *event = NULL;
     }
-    ext = extension_of(mt);
+    if (mc == NULL || (ext == NULL && stream == NULL)) {
+        return xccl_mem_component_reduce_multi(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, mt);
+    }
     if (ext == NULL) {
         return XCCL_ERR_NOT_IMPLEMENTED;
     }
-    return ext->reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, stream, event);
+    if (size == 0) {
+        return XCCL_OK;
+    }
+    st = ext->reduce_multi_nb(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, stream, event);
+    if (st == XCCL_ERR_NO_RESOURCE && stream == NULL) {
+        return mc->reduce_multi(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op);
+    }
+    if (st == XCCL_OK && event != NULL) {
+        (*event)->mem_type = mt;
+    }
+    return st;
 }
 
 /* reference mem_component.c:150-174: the first component, in memory-type

@@ -406,7 +406,6 @@ static xccl_status_t issue_reduce(ctx_t *c, rank_state_t *s, void *s1, void *s2,
                                   size_t stride)
 {
     const xccl_replay_params_t *p = c->p;
-    xccl_status_t               st;
 
     if (n2 == 0) {
         c->stats->reduce_calls++;
@@ -426,19 +425,15 @@ static xccl_status_t issue_reduce(ctx_t *c, rank_state_t *s, void *s1, void *s2,
         return n2 == 0 ? xccl_mem_component_reduce(s1, s2, out, count, p->dtype, p->op, MT)
                        : xccl_mem_component_reduce_multi(s1, s2, out, n2, count, stride, p->dtype, p->op, MT);
     }
-    if (count == 0) {
-        return XCCL_OK; /* nothing to launch, nothing to wait for */
-    }
-    st = n2 == 0 ? xccl_mem_component_reduce_nb(s1, s2, out, count, p->dtype, p->op, MT, NULL, &s->reduce_ev)
-                 : xccl_mem_component_reduce_multi_nb(s1, s2, out, n2, count, stride, p->dtype, p->op, MT, NULL,
-                                                      &s->reduce_ev);
-    if (st == XCCL_ERR_NO_RESOURCE) {
-        /* the component's event pool is empty (other collectives hold it): this reduction blocks */
-        s->reduce_ev = NULL;
-        st = n2 == 0 ? xccl_mem_component_reduce(s1, s2, out, count, p->dtype, p->op, MT)
-                     : xccl_mem_component_reduce_multi(s1, s2, out, n2, count, stride, p->dtype, p->op, MT);
-    }
-    return st;
+    /* As the patched call sites do (allreduce_knomial.c:74-80,129-135 and the
+     * other three files with integration/xccl-rocm.patch applied): one call,
+     * status ignored beyond passing it on; the dispatcher leaves the event
+     * NULL when the reduction is complete on return -- empty, or run through
+     * the blocking entry because the component's event pool was empty (other
+     * collectives hold it). */
+    return n2 == 0 ? xccl_mem_component_reduce_nb(s1, s2, out, count, p->dtype, p->op, MT, NULL, &s->reduce_ev)
+                   : xccl_mem_component_reduce_multi_nb(s1, s2, out, n2, count, stride, p->dtype, p->op, MT, NULL,
+                                                        &s->reduce_ev);
 }
 
 /* The "reduce in flight" phase: XCCL_OK once the result may be read. */

@@ -124,35 +124,53 @@ def component() -> RocmMemComponent:
     return RocmMemComponent.in_dll(component_lib(), "xccl_rocm_mem_component")
 
 
+def bind_dispatcher(path, mode=_c.DEFAULT_MODE):
+    """Loads a library that exports the xccl_mem_component_* dispatcher API
+    (reference src/utils/mem_component.h:52-95) and sets the argument types of
+    the entries it has: libxccl_mc.so, or a build of the reference's own
+    src/utils/mem_component.c (the *_nb entries exist there only with
+    integration/xccl-rocm.patch applied; event_wait / get only in libxccl_mc.so)."""
+    lib = _c.CDLL(path, mode=mode)
+    sigs = {
+        "xccl_mem_component_init": [_c.c_char_p],
+        "xccl_mem_component_alloc": [_c.POINTER(_vp), _sz, _int],
+        "xccl_mem_component_free": [_vp, _int],
+        "xccl_mem_component_type": [_vp, _c.POINTER(_int)],
+        "xccl_mem_component_reduce": [_vp, _vp, _vp, _sz, _int, _int, _int],
+        "xccl_mem_component_reduce_multi": [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _int],
+        "xccl_mem_component_reduce_nb": [_vp, _vp, _vp, _sz, _int, _int, _int, _c.POINTER(XcclStream),
+                                         _c.POINTER(_vp)],
+        "xccl_mem_component_reduce_multi_nb": [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _int,
+                                               _c.POINTER(XcclStream), _c.POINTER(_vp)],
+        "xccl_mem_component_memcpy_async": [_vp, _vp, _sz, _c.POINTER(XcclStream)],
+        "xccl_mem_component_start_acitivity": [_c.POINTER(XcclStream), _c.POINTER(_vp)],
+        "xccl_mem_component_finish_acitivity": [_vp],
+        "xccl_mc_event_record": [_c.POINTER(XcclStream), _c.POINTER(_vp)],
+        "xccl_mc_event_query": [_vp],
+        "xccl_mc_event_free": [_vp],
+        "xccl_mc_event_wait": [_vp],
+        "xccl_mem_component_free_cache": [],
+        "xccl_mem_component_finalize": [],
+        "xccl_mem_component_get": [_int],
+    }
+    for name, argtypes in sigs.items():
+        fn = getattr(lib, name, None)
+        if fn is None:
+            continue
+        fn.argtypes = argtypes
+        fn.restype = _ST
+    for name in ("xccl_mem_component_free_cache", "xccl_mem_component_finalize"):
+        getattr(lib, name).restype = None
+    if hasattr(lib, "xccl_mem_component_get"):
+        lib.xccl_mem_component_get.restype = _c.POINTER(MemComponentVtable)
+    return lib
+
+
 def dispatch_lib():
     global _dispatch_lib
     if _dispatch_lib is None:
         _need_built()
-        lib = _c.CDLL(DISPATCH_SO)
-        lib.xccl_mem_component_init.argtypes = [_c.c_char_p]
-        lib.xccl_mem_component_alloc.argtypes = [_c.POINTER(_vp), _sz, _int]
-        lib.xccl_mem_component_free.argtypes = [_vp, _int]
-        lib.xccl_mem_component_type.argtypes = [_vp, _c.POINTER(_int)]
-        lib.xccl_mem_component_reduce.argtypes = [_vp, _vp, _vp, _sz, _int, _int, _int]
-        lib.xccl_mem_component_reduce_multi.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _int]
-        lib.xccl_mem_component_reduce_nb.argtypes = [_vp, _vp, _vp, _sz, _int, _int, _int, _c.POINTER(XcclStream),
-                                                     _c.POINTER(_vp)]
-        lib.xccl_mem_component_reduce_multi_nb.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _int,
-                                                           _c.POINTER(XcclStream), _c.POINTER(_vp)]
-        lib.xccl_mem_component_memcpy_async.argtypes = [_vp, _vp, _sz, _c.POINTER(XcclStream)]
-        lib.xccl_mem_component_start_acitivity.argtypes = [_c.POINTER(XcclStream), _c.POINTER(_vp)]
-        lib.xccl_mem_component_finish_acitivity.argtypes = [_vp]
-        lib.xccl_mc_event_record.argtypes = [_c.POINTER(XcclStream), _c.POINTER(_vp)]
-        lib.xccl_mc_event_query.argtypes = [_vp]
-        lib.xccl_mc_event_free.argtypes = [_vp]
-        lib.xccl_mc_event_wait.argtypes = [_vp]
-        lib.xccl_mem_component_free_cache.argtypes = []
-        lib.xccl_mem_component_free_cache.restype = None
-        lib.xccl_mem_component_finalize.argtypes = []
-        lib.xccl_mem_component_finalize.restype = None
-        lib.xccl_mem_component_get.argtypes = [_int]
-        lib.xccl_mem_component_get.restype = _c.POINTER(MemComponentVtable)
-        _dispatch_lib = lib
+        _dispatch_lib = bind_dispatcher(DISPATCH_SO)
     return _dispatch_lib
 
 
