@@ -30,6 +30,9 @@ before the timed region.  Prints ONE JSON line.
                    reduce_multi_nb + hipStreamSynchronize, "graph" =
                    single-node hipGraph launch + hipStreamSynchronize,
                    "issue" = the host's cost of issuing one reduction
+  mid_sizes        the scatter-reduce regime (reference allreduce_sra.c:281-284):
+                   FLOAT32 SUM, 8 sources x 256 KiB .. 64 MiB per vector, kernel
+                   time (region-timed) beside the blocking call a caller sees
 """
 import argparse
 import json
@@ -200,6 +203,41 @@ def latency_sweep(mc, hip, iters, quick):
     return res, buf
 
 
+def mid_sizes(mc, hip):
+    """FLOAT32 SUM, 8 sources x 256 KiB .. 64 MiB per vector (powers of 4): average kernel duration (one event
+    pair around 200 back-to-back launches on the component's stream) and what a caller of the blocking entry
+    sees per call (host clock, p50 of 200 calls), both also as algorithmic GB/s."""
+    from xccl_amd.types import Dt, MemType, Op, Status
+    rows = {}
+    nsrc = 8
+    for vb in (256 << 10, 1 << 20, 4 << 20, 16 << 20, 64 << 20):
+        size = vb // 4
+        nb = (nsrc + 1) * vb
+        st, slab = mc.xccl_mem_component_alloc(nb, MemType.ROCM)
+        assert st == Status.OK, st
+        for j in range(nsrc):
+            assert mc.datagen_fill(slab + j * vb, size, Dt.FLOAT32, 4, j) == Status.OK
+        hip.device_synchronize()
+        region_gbps(mc, slab, nsrc, size, 4, Dt.FLOAT32, Op.SUM, 20)
+        g, us = region_gbps(mc, slab, nsrc, size, 4, Dt.FLOAT32, Op.SUM, 200)
+        route = mc.reduce_multi_route(slab, slab + vb, slab + nsrc * vb, nsrc - 1, size, vb, Dt.FLOAT32, Op.SUM, True)
+        if route["route"] == "stream":      # too large for the own queue: what the HIP stream path does with it
+            route = mc.reduce_multi_route(slab, slab + vb, slab + nsrc * vb, nsrc - 1, size, vb, Dt.FLOAT32, Op.SUM, False)
+            where = "hip stream"
+        else:
+            where = "own queue"
+        st, ns = mc.bench_latency("sync", slab, slab + vb, slab + nsrc * vb, nsrc - 1, size, vb, Dt.FLOAT32, Op.SUM, 220)
+        assert st == Status.OK, st
+        call_us = float(np.percentile(ns[20:], 50)) / 1e3
+        rows["n8_%dKiB" % (vb >> 10)] = {
+            "bytes_per_call": nb, "kernel_us": round(us, 2), "kernel_GBps": round(g, 1),
+            "blocking_call_us": round(call_us, 2), "blocking_call_p99_us": round(float(np.percentile(ns[20:], 99)) / 1e3, 2),
+            "blocking_call_GBps": round(nb / call_us / 1e3, 1), "call_minus_kernel_us": round(call_us - us, 2),
+            "launched_on": where, "completion": route["route"], "grid": route["grid"]}
+        mc.xccl_mem_component_free(slab, MemType.ROCM)
+    return rows
+
+
 def latency_extras(mc, hip, buf, iters):
     from xccl_amd.types import Dt, Op, Status
     res = {}
@@ -213,6 +251,18 @@ def latency_extras(mc, hip, buf, iters):
         ns = ns[:, iters // 10:]
         res["threads%d_n4_1024B" % th] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
                                           "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
+    # a small blocking call with a system-scope acquire fence on the own queue's packets instead of the agent-scope one
+    lib = mc.component_lib()
+    for scope, flag in (("agent", 0), ("system", 1)):
+        lib.xccl_rocm_set_direct_options(flag, -1, -1, -1, -1)
+        for nsrc, nbv in ((4, 1024), (8, 32768)):
+            st, ns = mc.bench_latency("sync", buf.ptr, buf.ptr + 32768, buf.ptr + 9 * 32768, nsrc - 1, nbv // 4, 32768,
+                                      Dt.FLOAT32, Op.SUM, iters)
+            assert st == Status.OK
+            ns = ns[iters // 10:]
+            res["acquire_%s_n%d_%dB" % (scope, nsrc, nbv)] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
+                                                              "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
+    lib.xccl_rocm_set_direct_options(0, -1, -1, -1, -1)
     tb.close()
     # memcpy_async + event_record + event_query: one message of the loopback transport / one mpod alltoall step
     ms = mc.Stream(hip.stream_create())
@@ -630,6 +680,7 @@ def main():
         lat.update(latency_extras(mc, hip, lbuf, min(a.latency_iters, 4000)))
         lbuf.close()
         out["latency_us"] = lat
+        out["mid_sizes"] = mid_sizes(mc, hip)
 
     print(json.dumps(out))
     return 0

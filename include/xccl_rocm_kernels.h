@@ -123,30 +123,79 @@ xccl_status_t xccl_rocm_reduce_multi_slots(void *sbuf1, void *sbuf2, void *rbuf,
  * xccl_rocm_reduce_multi_slots on the component's own dispatch queue instead
  * of a HIP stream, for callers that wait for the completion word and need no
  * stream order (the blocking entries of the vtable).  The launch goes out as
- * an AQL packet on one of two user-mode queues (`queue_slot` 0 or 1; any
- * other slot is not served) that the component creates through the HSA
- * runtime on first use; the host's part of the launch is writing the packet
- * and ringing the doorbell.  Launches of one queue run in order; they are not
- * ordered against any HIP stream: issue one only when everything it depends
- * on is complete, and wait for its completion word before anything depends on
- * it.
+ * an AQL packet on one of up to four user-mode queues (`queue_slot` 0..3; by
+ * default there are two, which slots 2 and 3 share with slots 0 and 1, see
+ * xccl_rocm_set_direct_options) that
+ * the component creates through the HSA runtime on first use; the host's part
+ * of the launch is writing the packet and ringing the doorbell.  Launches of
+ * one queue run in order, except that a `blocking` caller's launch -- the
+ * caller waits for it before it issues anything else -- may be allowed not to
+ * wait for other callers' launches on the same queue; they are not ordered
+ * against any HIP stream: issue one only when everything it depends on is
+ * complete, and wait for its completion before anything depends on it.
+ * `kernarg`: XCCL_ROCM_KERNARG_BYTES of pinned host memory that stay the
+ * caller's until the launch is complete (NULL: a ring of the queue's own,
+ * and the launch is ordered).
  * `*flagged` > 0: launched, complete when the first `*flagged` words at
- * `dev_flag` hold `seq`.  `*flagged` == 0 with XCCL_OK: nothing was launched
- * and the caller uses xccl_rocm_reduce_multi_slots instead -- the call is too
- * large to carry its own completion word (more than 6144 workgroups here;
- * XCCL_MC_ROCM_MAX_COUNTED_GRID), has size 0, the slot has no queue,
- * the queue could not be set up (said once on stderr), or the path is switched off
- * (XCCL_MC_ROCM_DIRECT_QUEUE=0 or xccl_rocm_set_direct_queue(0)).  Blocking
- * call, 4 sources x 32 KiB: p50 6.7 us against 7.6 us on a HIP stream, p99 7.0
- * against 11.3 us.  No counterpart in the reference.
+ * `dev_flag` hold `seq`.  `*flagged` == -1: launched, too large to count its
+ * own workgroups (more than 6144; XCCL_MC_ROCM_MAX_COUNTED_GRID): complete when
+ * xccl_rocm_direct_signal_done(*signal) -- `*signal` is created on first need
+ * (0 before) and belongs to the queues: it goes with
+ * xccl_rocm_direct_queue_destroy.  `*flagged` == 0 with XCCL_OK: nothing was
+ * launched and the caller uses xccl_rocm_reduce_multi_slots instead -- the
+ * call is too large and `signal` is NULL or that path is off, has size 0, the
+ * slot has no queue, the queue could not be set up (said once on stderr), or
+ * the path is switched off (XCCL_MC_ROCM_DIRECT_QUEUE=0 or
+ * xccl_rocm_set_direct_queue(0)).  Blocking call, 4 sources x 32 KiB: p50
+ * 6.7 us against 7.6 us on a HIP stream, p99 7.0 against 11.3 us.  No
+ * counterpart in the reference.
  */
+#define XCCL_ROCM_KERNARG_BYTES 128
 xccl_status_t xccl_rocm_reduce_multi_direct(void *sbuf1, void *sbuf2, void *rbuf,
                                             size_t count, size_t size,
                                             size_t stride, xccl_dt_t dtype,
                                             xccl_op_t op, int queue_slot,
                                             uint32_t *dev_count,
                                             uint32_t *dev_flag, uint32_t flag_words,
-                                            uint32_t seq, int *flagged);
+                                            uint32_t seq, uint64_t *signal,
+                                            void *kernarg, int blocking,
+                                            int *flagged);
+
+/* Nonzero once the launch that armed `signal` (see above) is complete. */
+int xccl_rocm_direct_signal_done(uint64_t signal);
+
+/*
+ * How the component's own queues are used; a negative (for `queues`: out of
+ * range) argument leaves that setting alone.  Each also has an environment
+ * variable, read once.
+ *   acquire_system  1: launches carry a system-scope acquire fence instead of
+ *                   an agent-scope one (XCCL_MC_ROCM_DIRECT_ACQUIRE=system)
+ *   queues          1..4 queues per device, for thread slots 0..queues-1
+ *                   (XCCL_MC_ROCM_DIRECT_QUEUES)
+ *   share           1 (default): the other thread slots share those queues;
+ *                   0: they keep to their HIP streams
+ *                   (XCCL_MC_ROCM_DIRECT_SHARE)
+ *   barrier         0 (default): a blocking caller's launch does not wait for
+ *                   other callers' launches on its queue; 1: every launch
+ *                   waits for all before it (XCCL_MC_ROCM_DIRECT_BARRIER)
+ *   signal          1: launches too large to count their own workgroups stay
+ *                   on these queues and complete through a completion signal;
+ *                   0 (default): they go to the HIP stream
+ *                   (XCCL_MC_ROCM_DIRECT_SIGNAL)
+ * Measured, blocking call, 4 sources x 1 KiB, p50 / p99 in us, 1 / 2 / 4
+ * calling threads: two queues shared, no barrier 5.5 / 5.8, 6.3 / 8.7,
+ * 6.7-7.2 / 13.2; shared, with barrier 6.3 / 7.1, 6.1-6.4 / 8.8, 6.9-7.7 /
+ * 13.6; two queues not shared (threads 3 and 4 on HIP streams) 5.4 / 5.8,
+ * 7.1-7.3 / 10.9, 10.1-10.6 / 30-32; four queues, no barrier 5.4-5.8 / 6.1,
+ * 6.1-6.4 / 9.0, 7.7 / 21; one queue shared by all 5.8-6.3 / 7.2, 6.6 / 8.9,
+ * 12.4-12.9 / 13.4.  A system-scope acquire costs 0.85 us on a 1 KiB call
+ * and 2.5 us on 8 sources x 32 KiB.  Completion by signal is no faster than
+ * the HIP stream with a queued one-lane kernel (8 sources x 16 MiB: 28.9-29.0
+ * against 28.4-28.8 us per blocking call, kernel 22.4; x 64 MiB: 96.8-97.0
+ * against 94.7-96.4, kernel 88.0).
+ */
+void xccl_rocm_set_direct_options(int acquire_system, int queues, int share,
+                                  int barrier, int signal);
 
 /* Launches that went out on the component's own queues so far (all devices). */
 uint64_t xccl_rocm_direct_launch_count(void);
@@ -158,8 +207,10 @@ int xccl_rocm_direct_queue_failed(void);
 /* Switches the path on or off for the process (default on). */
 void xccl_rocm_set_direct_queue(int on);
 
-/* Destroys the current device's queues and the code it loaded for them; no
- * launch may be in flight.  Called by the component's close(). */
+/* Destroys the current device's queues, their completion signals and the code
+ * loaded for them, after waiting (bounded: 10 s, or until a queue reports an
+ * error) for everything queued there to complete; the caller issues nothing
+ * more while it runs.  Called by the component's close(). */
 void xccl_rocm_direct_queue_destroy(void);
 
 /*
@@ -239,6 +290,13 @@ void xccl_rocm_set_burst_max_grid(int max_grid);
  * default (8).  For measurement and tests. */
 void xccl_rocm_set_slot_max_grid(int max_grid);
 
+/* Largest launch, in workgroups, that counts its own arrivals for the
+ * completion word: on a HIP stream (default 2048; larger ones get a one-lane
+ * kernel queued behind them) and on the component's own queue (default 6144).
+ * Negative = leave alone.  Also XCCL_MC_ROCM_MAX_COUNTED_GRID (sets both).
+ * For measurement and tests. */
+void xccl_rocm_set_counted_grid(int on_stream, int on_own_queue);
+
 /* What a launch with these arguments would be: grid/block size and the
  * mangled kernel name (truncated into `name`, if not NULL).  Host-only apart
  * from the CU-count query.  Returns the status the launch would return. */
@@ -248,6 +306,27 @@ xccl_status_t xccl_rocm_reduce_multi_plan(void *sbuf1, void *sbuf2, void *rbuf,
                                           xccl_op_t op, unsigned *grid,
                                           unsigned *block, char *name,
                                           size_t name_len);
+
+/* What a launch with these arguments, asked to report its own completion,
+ * would be -- on a HIP stream (`own_queue` 0) or on the component's own queue
+ * (1): grid in workgroups, bytes of LDS asked for to bound the resident
+ * workgroups per compute unit (0: no bound), whether it runs the burst
+ * kernel, and how the host learns that it is complete.  Any output may be
+ * NULL.  Host-only apart from the CU-count query; every launch-shape knob and
+ * its environment variable shows here.  For tests. */
+enum {
+    XCCL_ROCM_ROUTE_STREAM  = 0, /* no completion word: the caller waits for the stream */
+    XCCL_ROCM_ROUTE_SLOTS   = 1, /* one word per workgroup */
+    XCCL_ROCM_ROUTE_COUNTED = 2, /* the last workgroup to arrive writes the word */
+    XCCL_ROCM_ROUTE_TAIL    = 3, /* a one-lane kernel queued behind the launch writes it */
+    XCCL_ROCM_ROUTE_SIGNAL  = 4  /* the packet's completion signal (own queue only) */
+};
+xccl_status_t xccl_rocm_reduce_multi_route(void *sbuf1, void *sbuf2, void *rbuf,
+                                           size_t count, size_t size,
+                                           size_t stride, xccl_dt_t dtype,
+                                           xccl_op_t op, int own_queue,
+                                           unsigned *grid, unsigned *lds_bytes,
+                                           int *burst, int *route);
 
 /*
  * Stream gate used by start/finish_stream_activity: one wave polls the

@@ -25,6 +25,13 @@ def test_mem_type_probe(rocm):
     assert rocm.xccl_mem_component_type(d.ptr + 512) == (Status.OK, MemType.ROCM)
     pinned = hip.host_malloc(1024)
     assert rocm.xccl_mem_component_type(pinned) == (Status.OK, MemType.HOST)
+    # managed memory is not "Device" to the runtime: HOST, like in the reference (cuda_mem_component.c:198-202)
+    managed = hip.malloc_managed(1 << 16)
+    assert rocm.xccl_mem_component_type(managed) == (Status.OK, MemType.HOST)
+    assert rocm.xccl_mem_component_type(managed + 12345) == (Status.OK, MemType.HOST)
+    mt = ctypes.c_int(-1)
+    assert rocm.component().super.mem_type(managed + 4096, ctypes.byref(mt)) == Status.OK and mt.value == MemType.HOST
+    hip.free(managed)
     plain = ctypes.create_string_buffer(64)
     assert rocm.xccl_mem_component_type(ctypes.addressof(plain)) == (Status.OK, MemType.HOST)
     mt = ctypes.c_int(-1)
@@ -782,9 +789,11 @@ def test_first_use_of_a_device_inside_a_capture_is_refused():
 
 def test_component_works_again_after_close():
     """close() releases a device's streams, events, dispatch queues and the
-    code loaded for them; the next call sets everything up again.  A fresh
-    process: reductions on the own queue and on the stream, close (through the
-    dispatcher's free_cache), the same reductions once more."""
+    code loaded for them -- after everything queued there has completed, also
+    launches whose event nobody waited for; the next call sets everything up
+    again.  A fresh process: reductions on the own queue and on the stream,
+    four unwaited ones, close (through the dispatcher's free_cache), the same
+    reductions once more."""
     import os
     import subprocess
     import sys
@@ -810,7 +819,14 @@ def test_component_works_again_after_close():
         "    got = buf.download(np.float32, count, 2 * n * 4)\n"
         "    return int(st), int(lib.xccl_rocm_direct_launch_count() - before), bool((got == want[:count]).all())\n"
         "a = [run(1000), run(1000), run(n)]\n"
+        "# launches nobody waits for, on the own queue and on the stream, are still in flight when the component closes\n"
+        "for count in (1000, n // 2, 1000, n):\n"
+        "    st, ev = mc.xccl_mem_component_reduce_multi_nb(buf.ptr, buf.ptr + n * 4, buf.ptr + 2 * n * 4, 1, count, n * 4,\n"
+        "                                                   Dt.FLOAT32, Op.SUM, MemType.ROCM, None)\n"
+        "    assert st == Status.OK and ev\n"
         "mc.xccl_mem_component_free_cache()\n"
+        "got = buf.download(np.float32, n, 2 * n * 4)\n"
+        "assert (got == want).all(), 'close() did not wait for the launches in flight'\n"
         "b = [run(1000), run(1000), run(n)]\n"
         "print('before', a, 'after', b)\n"
     ) % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))

@@ -91,7 +91,7 @@ def test_static_scratch_entry_matches_flagged_entry(rocm, oracle):
 
 def test_static_scratch_entry_limits(rocm):
     """More than 8192 workgroups (8 MiB per vector) is refused before anything is enqueued; so is a call
-    without a completion word; an unsupported pair and a zero size behave as in the other entries."""
+    without a completion word; an unsupported pair is refused; a zero size reduces nothing and still writes the word."""
     lib = rocm.component_lib()
     stream = rocm.component_stream()
     host_word = hip.host_malloc(64)
@@ -106,9 +106,23 @@ def test_static_scratch_entry_limits(rocm):
         hip.stream_synchronize(stream)
         assert ctypes.cast(host_word, ctypes.POINTER(ctypes.c_uint32))[0] == 0
         small = (buf, buf + n * 4, buf + 2 * n * 4, 1, 0, n * 4, int(Dt.FLOAT32), int(Op.SUM), stream)
-        assert lib.xccl_rocm_reduce_multi_flagged_static(*small, dev_word, 2) == Status.OK          # size 0: no-op
+        # size 0: nothing to reduce, but a caller polling the word must not wait in vain -- it is written, in stream order
+        hip.memset(buf + 2 * n * 4, 0x5A, 64)
+        assert lib.xccl_rocm_reduce_multi_flagged_static(*small, dev_word, 2) == Status.OK
+        word = ctypes.cast(host_word, ctypes.POINTER(ctypes.c_uint32))
+        t0 = time.time()
+        while word[0] != 2:
+            assert time.time() - t0 < 20.0, "size == 0: the completion word was never written"
+        hip.stream_synchronize(stream)
+        probe = np.empty(64, dtype=np.uint8)
+        hip.memcpy_dtoh(probe, buf + 2 * n * 4)
+        assert (probe == 0x5A).all()                                                                # and nothing else is
         bad = (buf, buf + n * 4, buf + 2 * n * 4, 1, 16, n * 4, int(Dt.FLOAT32), int(Op.BAND), stream)
         assert lib.xccl_rocm_reduce_multi_flagged_static(*bad, dev_word, 3) == Status.ERR_UNSUPPORTED
+        bad0 = (buf, buf + n * 4, buf + 2 * n * 4, 1, 0, n * 4, int(Dt.FLOAT32), int(Op.BAND), stream)
+        assert lib.xccl_rocm_reduce_multi_flagged_static(*bad0, dev_word, 4) == Status.ERR_UNSUPPORTED
+        hip.stream_synchronize(stream)
+        assert word[0] == 2
     finally:
         hip.free(buf)
         hip.host_free(host_word)

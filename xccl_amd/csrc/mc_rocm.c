@@ -74,7 +74,9 @@ typedef struct mc_rocm_event {
     xccl_mc_event_t    super;
     atomic_int         is_free;
     hipEvent_t         hip_event;
-    int                flagged;   /* n > 0: done when the first n words at flag all equal expect */
+    int                flagged;   /* n > 0: done when the first n words at flag all equal expect; -1: when `signal` reads 0 */
+    uint64_t           signal;    /* completion signal of the own dispatch queue, created when first needed (0: none yet) */
+    void              *kernarg;   /* kernel-argument block for launches on the own dispatch queue (pinned host memory) */
     uint32_t           expect;    /* last sequence number handed to a kernel */
     volatile uint32_t *flag;      /* host view of the completion word */
     uint32_t          *dev_flag;  /* device view of the same word */
@@ -115,6 +117,7 @@ typedef struct mc_rocm_device {
     int                     *gate_words;  /* pinned, mapped */
     uint32_t                *flag_words; /* pinned, mapped: completion words of the events */
     uint32_t                *arrival_counts; /* device */
+    char                    *kernargs;       /* pinned: XCCL_ROCM_KERNARG_BYTES per event */
     /* Launches put on each reduction stream, and the highest of them known to be complete (the stream runs
      * them in order).  While the two differ, the stream may hold work nobody has waited for, and a call of that
      * slot stays on the stream, behind it, instead of taking the component's own dispatch queue. */
@@ -224,6 +227,9 @@ static void mc_rocm_device_destroy(mc_rocm_device_t *d)
     if (d->arrival_counts != NULL) {
         (void)hipFree(d->arrival_counts);
     }
+    if (d->kernargs != NULL) {
+        (void)hipHostFree(d->kernargs);
+    }
     for (i = 0; i < MC_NUM_STREAMS; i++) {
         if (d->stream[i] != NULL) {
             (void)hipStreamDestroy(d->stream[i]);
@@ -258,8 +264,12 @@ static xccl_status_t mc_rocm_device_create_parts(mc_rocm_device_t *d)
     MC_HIP(hipMemsetAsync(d->arrival_counts, 0,
                           XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_DONE_COUNT_BYTES, d->stream[0]));
     MC_HIP(hipStreamSynchronize(d->stream[0]));
+    MC_HIP(hipHostMalloc((void **)&d->kernargs, XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_KERNARG_BYTES, hipHostMallocDefault));
+    memset(d->kernargs, 0, XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_KERNARG_BYTES);
     for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
         mc_rocm_event_t *ev = &d->events[i];
+        ev->kernarg = d->kernargs + (size_t)i * XCCL_ROCM_KERNARG_BYTES;
+        ev->signal  = 0;
         MC_HIP(hipEventCreateWithFlags(&ev->hip_event, hipEventDisableTiming));
         ev->flag = &d->flag_words[i * MC_FLAG_STRIDE];
         MC_HIP(hipHostGetDevicePointer((void **)&ev->dev_flag, (void *)ev->flag, 0));
@@ -454,8 +464,9 @@ static xccl_status_t mc_rocm_mem_type(void *ptr, ucs_memory_type_t *mem_type)
  * small stream-ordered reduction followed by a large one). */
 static _Thread_local struct {
     volatile uint32_t *flag;
-    int                words;
+    int                words; /* -1: complete when `signal` reads 0 */
     uint32_t           expect;
+    uint64_t           signal;
     unsigned           generation;
 } mc_last_direct;
 
@@ -473,6 +484,13 @@ static void mc_rocm_wait_last_direct(void)
     if (mc_last_direct.generation != atomic_load(&mc_generation)) {
         mc_last_direct.flag = NULL;
         return;
+    }
+    while (mc_last_direct.words < 0 && !xccl_rocm_direct_signal_done(mc_last_direct.signal)) {
+        /* (a later launch of the same event re-arms the signal only after this one was seen complete) */
+        if ((++polls & 0xffffu) == 0 && xccl_rocm_direct_queue_failed()) {
+            break;
+        }
+        MC_CPU_RELAX();
     }
     for (i = 0; i < mc_last_direct.words; i++) {
         /* sequence numbers of a word only grow: at or past ours means ours is done */
@@ -511,6 +529,9 @@ static int mc_rocm_flag_done(const mc_rocm_event_t *ev)
 {
     int i;
 
+    if (ev->flagged < 0) {
+        return xccl_rocm_direct_signal_done(ev->signal);
+    }
     for (i = 0; i < ev->flagged; i++) {
         if (__atomic_load_n(&ev->flag[i], __ATOMIC_ACQUIRE) != ev->expect) {
             return 0;
@@ -642,6 +663,8 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
                                            stride, dtype, op, slot,
                                            ev->dev_count, ev->dev_flag,
                                            MC_FLAG_STRIDE, ev->expect + 1,
+                                           &ev->signal, ev->kernarg,
+                                           want_sync && mc_last_direct.flag == NULL,
                                            &flagged);
         if (st != XCCL_OK) {
             atomic_store(&ev->is_free, MC_SLOT_FREE);
@@ -653,13 +676,16 @@ static xccl_status_t mc_rocm_do_reduce_multi(void *sbuf1, void *sbuf2,
             ev->direct  = 1;
             ev->slot    = -1;
             ev->polls   = 0;
-            ev->expect++;
+            if (flagged > 0) {
+                ev->expect++;
+            }
             if (want_sync) {
                 st = mc_rocm_flag_poll(ev, 1);
             } else {
                 mc_last_direct.flag       = ev->flag;
                 mc_last_direct.words      = flagged;
                 mc_last_direct.expect     = ev->expect;
+                mc_last_direct.signal     = ev->signal;
                 mc_last_direct.generation = atomic_load(&mc_generation);
             }
             if (event != NULL && st == XCCL_OK) {

@@ -11,6 +11,7 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <vector>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -37,6 +38,8 @@ constexpr size_t kLdsPerGroup   = 64 * 1024; // most a workgroup may ask for
 // completion signal up to here and would serialise a grid of hundreds of
 // thousands.
 constexpr unsigned kMaxFlaggedGrid = 8192;
+// Hard bound of what XCCL_MC_ROCM_MAX_COUNTED_GRID may ask for (measurement; the two-level count itself has no limit).
+constexpr unsigned kMaxCountedGridKnob = 1u << 20;
 
 std::atomic<int> g_blocks_per_cu{-1}; // -1: not read from the environment yet
 std::atomic<int> g_resident{0};
@@ -80,7 +83,7 @@ void read_env_once()
         g_slot_max_grid.store((unsigned)atoi(smg), std::memory_order_release);
     }
     const char *mcg = getenv("XCCL_MC_ROCM_MAX_COUNTED_GRID");
-    if (mcg != nullptr && atoi(mcg) >= 0 && (unsigned)atoi(mcg) <= kMaxFlaggedGrid) {
+    if (mcg != nullptr && atoi(mcg) >= 0 && (unsigned)atoi(mcg) <= kMaxCountedGridKnob) {
         g_max_counted_grid.store((unsigned)atoi(mcg), std::memory_order_release);
         g_direct_counted_grid.store((unsigned)atoi(mcg), std::memory_order_release);
     }
@@ -552,15 +555,40 @@ __global__ void clear_words_kernel(uint32_t *p, uint32_t n)
 }
 
 
-// Arms `plan` to write its own completion word; returns how many words the
-// host has to watch (one word per workgroup for a handful of workgroups, else
-// the first word, written by the last workgroup to arrive).
-int arm_completion(Plan &plan, uint32_t *dev_count, uint32_t *dev_flag, uint32_t flag_words, uint32_t seq)
+// How the host learns that a launch is complete (values of XCCL_ROCM_ROUTE_*):
+// one word per workgroup for a handful of workgroups, a word written by the
+// last workgroup to arrive for small grids, and for larger ones a one-lane
+// kernel queued behind the launch on a HIP stream or the packet's completion
+// signal on the component's own queue; else the stream itself.
+std::atomic<int> *direct_signal_knob();
+
+int completion_route(const Plan &plan, uint32_t flag_words, bool own_queue, bool want_flag, bool has_signal)
 {
-    // a grid of one needs neither counting nor a second word: it stays on the counting path, which then has no atomics
+    if (!want_flag) {
+        return XCCL_ROCM_ROUTE_STREAM;
+    }
+    const bool     tail_ok   = g_tail_flag.load(std::memory_order_relaxed) != 0;
+    const unsigned counted   = own_queue ? g_direct_counted_grid.load(std::memory_order_relaxed)
+                               : tail_ok ? g_max_counted_grid.load(std::memory_order_relaxed)
+                                         : kMaxFlaggedGrid;
     const unsigned slots_max = flag_words < XCCL_ROCM_FLAG_WORDS ? flag_words : XCCL_ROCM_FLAG_WORDS;
-    const bool     by_slots  = plan.grid > 1 && plan.grid <= slots_max &&
-                               plan.grid <= g_slot_max_grid.load(std::memory_order_relaxed);
+    if (plan.grid <= counted) {
+        // a grid of one needs neither counting nor a second word: it stays on the counting path, which then has no atomics
+        const bool by_slots = plan.grid > 1 && plan.grid <= slots_max && plan.grid <= g_slot_max_grid.load(std::memory_order_relaxed);
+        return by_slots ? XCCL_ROCM_ROUTE_SLOTS : XCCL_ROCM_ROUTE_COUNTED;
+    }
+    if (own_queue) {
+        return has_signal && direct_signal_knob()->load(std::memory_order_relaxed) != 0 ? XCCL_ROCM_ROUTE_SIGNAL
+                                                                                         : XCCL_ROCM_ROUTE_STREAM;
+    }
+    return tail_ok ? XCCL_ROCM_ROUTE_TAIL : XCCL_ROCM_ROUTE_STREAM;
+}
+
+// Arms `plan` to write its own completion word (route SLOTS or COUNTED);
+// returns how many words the host has to watch.
+int arm_completion(Plan &plan, int route, uint32_t *dev_count, uint32_t *dev_flag, uint32_t seq)
+{
+    const bool by_slots = route == XCCL_ROCM_ROUTE_SLOTS;
     plan.args.done_seq   = seq;
     plan.args.done_count = dev_count;
     plan.args.done_slots = by_slots ? plan.grid : 0;
@@ -595,7 +623,8 @@ extern const unsigned char *const xccl_rocm_kernel_image_begin[5];
 extern const unsigned char *const xccl_rocm_kernel_image_end[5];
 }
 
-constexpr int      kDirectQueues  = 2;
+constexpr int      kMaxDirectQueues = 4; // one per thread slot at most
+constexpr int      kDefaultDirectQueues = 2;
 constexpr uint32_t kDirectPackets = 256; // queue size; a blocking caller has one launch in flight
 constexpr size_t   kKernargSlot   = 128; // >= sizeof(ReduceArgs), one cache line pair per packet
 // Twice as many argument slots as packets: a packet is written once the queue has *consumed* the one 256
@@ -603,6 +632,7 @@ constexpr size_t   kKernargSlot   = 128; // >= sizeof(ReduceArgs), one cache lin
 // 256 behind its last user has been consumed, and the barrier bit makes that wait for everything before it.
 constexpr uint32_t kKernargSlots  = 2 * kDirectPackets;
 static_assert(sizeof(ReduceArgs) <= kKernargSlot, "kernel argument slot");
+static_assert(XCCL_ROCM_KERNARG_BYTES == kKernargSlot, "kernel argument block a caller brings");
 
 struct DirectKernel {
     uint64_t object = 0; // kernel descriptor address
@@ -624,7 +654,8 @@ struct DirectDevice {
     int                                           readers = 0;
     bool                                          hsa_up  = false;
     std::unordered_map<const void *, DirectKernel> kernels; // by HIP function pointer
-    DirectQueue                                   queue[kDirectQueues];
+    DirectQueue                                   queue[kMaxDirectQueues];
+    std::vector<hsa_signal_t>                     signals; // completion signals handed out, destroyed with the queues
 };
 
 DirectDevice          g_direct[kMaxDevices];
@@ -632,11 +663,53 @@ std::atomic<int>      g_direct_enabled{-1}; // -1: environment not read yet
 std::atomic<int>      g_direct_failed{0};   // a queue reported an error: launches on it may never complete
 std::atomic<uint64_t> g_direct_launches{0};
 
+// How the component's own queues are used (environment, read with XCCL_MC_ROCM_DIRECT_QUEUE; setters below):
+//   g_direct_acquire  scope of the acquire fence in front of a launch: agent (what HIP gives a kernel that
+//                     follows other kernels) or system (XCCL_MC_ROCM_DIRECT_ACQUIRE=system)
+//   g_direct_queues   queues per device, one per thread slot from slot 0 up (XCCL_MC_ROCM_DIRECT_QUEUES, 1..4)
+//   g_direct_share    1: thread slots beyond the last queue share the queues round-robin instead of keeping to
+//                     their HIP streams (XCCL_MC_ROCM_DIRECT_SHARE)
+//   g_direct_barrier  0: a blocking call's packet does not carry the barrier bit, i.e. does not wait for other
+//                     threads' launches on the same queue (XCCL_MC_ROCM_DIRECT_BARRIER)
+//   g_direct_signal   1: launches too large to count their own workgroups stay on the own queue and complete
+//                     through a completion signal on their packet (XCCL_MC_ROCM_DIRECT_SIGNAL)
+std::atomic<uint32_t> g_direct_acquire{HSA_FENCE_SCOPE_AGENT};
+std::atomic<int>      g_direct_queues{kDefaultDirectQueues};
+std::atomic<int>      g_direct_share{1};
+std::atomic<int>      g_direct_barrier{0};
+std::atomic<int>      g_direct_signal{0};
+
+std::atomic<int> *direct_signal_knob()
+{
+    return &g_direct_signal;
+}
+
 bool direct_enabled()
 {
     int on = g_direct_enabled.load(std::memory_order_acquire);
     if (on < 0) {
         const char *e = getenv("XCCL_MC_ROCM_DIRECT_QUEUE");
+        const char *a = getenv("XCCL_MC_ROCM_DIRECT_ACQUIRE");
+        const char *n = getenv("XCCL_MC_ROCM_DIRECT_QUEUES");
+        const char *h = getenv("XCCL_MC_ROCM_DIRECT_SHARE");
+        const char *b = getenv("XCCL_MC_ROCM_DIRECT_BARRIER");
+        const char *g = getenv("XCCL_MC_ROCM_DIRECT_SIGNAL");
+        if (a != nullptr) {
+            g_direct_acquire.store(strcmp(a, "system") == 0 ? HSA_FENCE_SCOPE_SYSTEM : HSA_FENCE_SCOPE_AGENT,
+                                   std::memory_order_release);
+        }
+        if (n != nullptr && atoi(n) >= 1 && atoi(n) <= kMaxDirectQueues) {
+            g_direct_queues.store(atoi(n), std::memory_order_release);
+        }
+        if (h != nullptr) {
+            g_direct_share.store(atoi(h) != 0, std::memory_order_release);
+        }
+        if (b != nullptr) {
+            g_direct_barrier.store(atoi(b) != 0, std::memory_order_release);
+        }
+        if (g != nullptr) {
+            g_direct_signal.store(atoi(g) != 0, std::memory_order_release);
+        }
         on = (e == nullptr || atoi(e) != 0) ? 1 : 0;
         g_direct_enabled.store(on, std::memory_order_release);
     }
@@ -823,18 +896,31 @@ DirectDevice *direct_device()
     return state == 1 ? &dd : nullptr;
 }
 
-// Puts `plan` on queue `slot` of the current device.  Anything but XCCL_OK:
-// nothing was enqueued and the caller launches on a HIP stream instead.
-xccl_status_t direct_launch(int slot, const Plan &plan)
+// A completion signal for launches of the current device's queues (destroyed
+// with the queues).  Nothing waits on it through the runtime -- the host reads
+// its value -- so it needs no interrupt.
+bool direct_signal_create(DirectDevice &dd, uint64_t *handle)
 {
-    if (slot < 0 || slot >= kDirectQueues) {
+    std::lock_guard<std::mutex> guard(dd.lock);
+    hsa_signal_t                sig{};
+    if (hsa_amd_signal_create(0, 0, nullptr, HSA_AMD_SIGNAL_AMD_GPU_ONLY, &sig) != HSA_STATUS_SUCCESS || sig.handle == 0) {
+        return false;
+    }
+    dd.signals.push_back(sig);
+    *handle = sig.handle;
+    return true;
+}
+
+// Puts `plan` on queue `slot` of the current device.  `signal` != 0: the packet
+// processor sets that signal to 0 when the launch is complete (the caller set
+// nothing: it is armed here).  `ordered`: the launch waits for everything
+// queued before it.  Anything but XCCL_OK: nothing was enqueued and the caller
+// launches on a HIP stream instead.
+xccl_status_t direct_launch(DirectDevice &dd, int slot, const Plan &plan, uint64_t signal, bool ordered, void *kernarg)
+{
+    if (slot < 0 || slot >= kMaxDirectQueues) {
         return XCCL_ERR_NO_RESOURCE;
     }
-    DirectDevice *found = direct_device();
-    if (found == nullptr) {
-        return XCCL_ERR_NO_RESOURCE;
-    }
-    DirectDevice &dd = *found;
     DirectKernel k;
     DirectQueue *dq = nullptr;
     if (!direct_kernel(dd, plan.fn, &k) || !direct_queue(dd, slot, &dq)) {
@@ -853,7 +939,8 @@ xccl_status_t direct_launch(int slot, const Plan &plan)
             return XCCL_ERR_NO_RESOURCE; // the queue is dead; the reserved packet stays invalid
         }
     }
-    char *args = dq->kernarg + (idx & (kKernargSlots - 1)) * kKernargSlot;
+    // the caller's own argument block (its until the launch is complete), else the queue's ring
+    char *args = kernarg != nullptr ? static_cast<char *>(kernarg) : dq->kernarg + (idx & (kKernargSlots - 1)) * kKernargSlot;
     memcpy(args, &plan.args, sizeof(ReduceArgs));
 
     hsa_kernel_dispatch_packet_t *p = static_cast<hsa_kernel_dispatch_packet_t *>(q->base_address) + (idx & (q->size - 1));
@@ -869,10 +956,13 @@ xccl_status_t direct_launch(int slot, const Plan &plan)
     p->kernel_object        = k.object;
     p->kernarg_address      = args;
     p->reserved2            = 0;
-    p->completion_signal.handle = 0; // completion is the kernel's own word
+    p->completion_signal.handle = signal; // 0: completion is the kernel's own word
+    if (signal != 0) {
+        hsa_signal_store_relaxed(hsa_signal_t{signal}, 1);
+    }
     const uint32_t header = (uint32_t)HSA_PACKET_TYPE_KERNEL_DISPATCH << HSA_PACKET_HEADER_TYPE |
-                            1u << HSA_PACKET_HEADER_BARRIER |
-                            (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE |
+                            (ordered ? 1u : 0u) << HSA_PACKET_HEADER_BARRIER |
+                            g_direct_acquire.load(std::memory_order_relaxed) << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE |
                             (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE;
     const uint32_t setup  = 1u << HSA_KERNEL_DISPATCH_PACKET_SETUP_DIMENSIONS;
     // header and setup share the packet's first 32-bit word: one release store makes the packet valid
@@ -882,13 +972,54 @@ xccl_status_t direct_launch(int slot, const Plan &plan)
     return XCCL_OK;
 }
 
-// Releases the queues and the executable of one device.  The caller has made
-// sure no launch is in flight (blocking callers have returned).
+// Waits until everything queued on `q` has completed: a barrier packet with a
+// completion signal goes in behind it (a stream-ordered launch whose event
+// nobody waited for may still be queued or running when the component closes).
+// Bounded: gives up after `limit_ns`, or when the queue has reported an error.
+void direct_drain(hsa_queue_t *q, uint64_t limit_ns)
+{
+    hsa_signal_t done{};
+    if (g_direct_failed.load(std::memory_order_acquire) != 0 ||
+        hsa_amd_signal_create(1, 0, nullptr, HSA_AMD_SIGNAL_AMD_GPU_ONLY, &done) != HSA_STATUS_SUCCESS) {
+        return;
+    }
+    const uint64_t t0  = clock_ns();
+    const uint64_t idx = hsa_queue_add_write_index_scacq_screl(q, 1);
+    bool           room = true;
+    while (idx - hsa_queue_load_read_index_scacquire(q) >= q->size) {
+        if (g_direct_failed.load(std::memory_order_acquire) != 0 || clock_ns() - t0 > limit_ns) {
+            room = false; // the reserved packet stays invalid; the queue is about to be destroyed anyway
+            break;
+        }
+    }
+    if (room) {
+        hsa_barrier_and_packet_t *b = static_cast<hsa_barrier_and_packet_t *>(q->base_address) + (idx & (q->size - 1));
+        memset(reinterpret_cast<char *>(b) + 4, 0, sizeof(*b) - 4);
+        b->completion_signal = done;
+        const uint32_t header = (uint32_t)HSA_PACKET_TYPE_BARRIER_AND << HSA_PACKET_HEADER_TYPE |
+                                1u << HSA_PACKET_HEADER_BARRIER |
+                                (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE |
+                                (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE;
+        __atomic_store_n(reinterpret_cast<uint32_t *>(b), header, __ATOMIC_RELEASE);
+        hsa_signal_store_screlease(q->doorbell_signal, (hsa_signal_value_t)idx);
+        while (hsa_signal_load_scacquire(done) != 0) {
+            if (g_direct_failed.load(std::memory_order_acquire) != 0 || clock_ns() - t0 > limit_ns) {
+                fprintf(stderr, "xccl mc_rocm: the component's dispatch queue did not drain; destroying it anyway\n");
+                break;
+            }
+        }
+    }
+    (void)hsa_signal_destroy(done);
+}
+
+// Releases the queues and the executable of one device, after everything
+// queued there has completed.
 void direct_destroy(DirectDevice &dd)
 {
     std::lock_guard<std::mutex> guard(dd.lock);
     for (DirectQueue &dq : dd.queue) {
         if (dq.q != nullptr) {
+            direct_drain(dq.q, 10000000000ull);
             (void)hsa_queue_destroy(dq.q);
             dq.q = nullptr;
         }
@@ -897,6 +1028,10 @@ void direct_destroy(DirectDevice &dd)
             dq.kernarg = nullptr;
         }
     }
+    for (hsa_signal_t sig : dd.signals) {
+        (void)hsa_signal_destroy(sig);
+    }
+    dd.signals.clear();
     dd.kernels.clear();
     dd.generation.fetch_add(1, std::memory_order_release); // kernel descriptors cached by the threads are stale now
     if (dd.exe.handle != 0) {
@@ -964,7 +1099,7 @@ xccl_status_t xccl_rocm_reduce_multi_flagged(void *sbuf1, void *sbuf2, void *rbu
 xccl_status_t xccl_rocm_reduce_multi_direct(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
                                             size_t stride, xccl_dt_t dtype, xccl_op_t op, int queue_slot,
                                             uint32_t *dev_count, uint32_t *dev_flag, uint32_t flag_words, uint32_t seq,
-                                            int *flagged)
+                                            uint64_t *signal, void *kernarg, int blocking, int *flagged)
 {
     if (flagged == nullptr || dev_count == nullptr || dev_flag == nullptr) {
         return XCCL_ERR_INVALID_PARAM;
@@ -976,15 +1111,77 @@ xccl_status_t xccl_rocm_reduce_multi_direct(void *sbuf1, void *sbuf2, void *rbuf
     if (st != XCCL_OK || nothing) {
         return st;
     }
-    if (plan.grid > g_direct_counted_grid.load(std::memory_order_relaxed) || plan.grid > kMaxFlaggedGrid) {
-        return XCCL_OK; // completes through the stream: not for this queue
+    DirectDevice *dd = direct_device();
+    if (dd == nullptr || queue_slot < 0) {
+        return XCCL_OK; // the caller takes the stream path
     }
-    const int words = arm_completion(plan, dev_count, dev_flag, flag_words, seq);
-    if (direct_launch(queue_slot, plan) != XCCL_OK) {
+    const int queues = g_direct_queues.load(std::memory_order_relaxed);
+    if (queue_slot >= queues) {
+        if (g_direct_share.load(std::memory_order_relaxed) == 0) {
+            return XCCL_OK; // this thread slot keeps to its HIP stream
+        }
+        queue_slot %= queues;
+    }
+    // A blocking caller has waited for its own earlier launches: its packet need not wait for other threads'.
+    // Such a packet may still be running when the queue's argument ring comes round again, so it must bring
+    // an argument block of its own.
+    const bool ordered  = blocking == 0 || kernarg == nullptr || g_direct_barrier.load(std::memory_order_relaxed) != 0;
+    const int route = completion_route(plan, flag_words, true, true, signal != nullptr);
+    if (route == XCCL_ROCM_ROUTE_STREAM) {
+        return XCCL_OK; // too many workgroups to count themselves: the launch completes through the stream
+    }
+    if (route == XCCL_ROCM_ROUTE_SIGNAL) {
+        if (*signal == 0 && !direct_signal_create(*dd, signal)) {
+            return XCCL_OK;
+        }
+        if (direct_launch(*dd, queue_slot, plan, *signal, ordered, kernarg) == XCCL_OK) {
+            *flagged = -1;
+        }
+        return XCCL_OK;
+    }
+    const int words = arm_completion(plan, route, dev_count, dev_flag, seq);
+    if (direct_launch(*dd, queue_slot, plan, 0, ordered, kernarg) != XCCL_OK) {
         return XCCL_OK; // not launched: the caller takes the stream path
     }
     *flagged = words;
     return XCCL_OK;
+}
+
+int xccl_rocm_direct_signal_done(uint64_t signal)
+{
+    return hsa_signal_load_scacquire(hsa_signal_t{signal}) == 0;
+}
+
+void xccl_rocm_set_counted_grid(int on_stream, int on_own_queue)
+{
+    read_env_once();
+    if (on_stream >= 0 && (unsigned)on_stream <= kMaxCountedGridKnob) {
+        g_max_counted_grid.store((unsigned)on_stream, std::memory_order_release);
+    }
+    if (on_own_queue >= 0 && (unsigned)on_own_queue <= kMaxCountedGridKnob) {
+        g_direct_counted_grid.store((unsigned)on_own_queue, std::memory_order_release);
+    }
+    g_shape_epoch.fetch_add(1, std::memory_order_release);
+}
+
+void xccl_rocm_set_direct_options(int acquire_system, int queues, int share, int barrier, int signal)
+{
+    (void)direct_enabled(); // environment first, so that it does not overwrite these later
+    if (acquire_system >= 0) {
+        g_direct_acquire.store(acquire_system ? HSA_FENCE_SCOPE_SYSTEM : HSA_FENCE_SCOPE_AGENT, std::memory_order_release);
+    }
+    if (queues >= 1 && queues <= kMaxDirectQueues) {
+        g_direct_queues.store(queues, std::memory_order_release);
+    }
+    if (share >= 0) {
+        g_direct_share.store(share != 0, std::memory_order_release);
+    }
+    if (barrier >= 0) {
+        g_direct_barrier.store(barrier != 0, std::memory_order_release);
+    }
+    if (signal >= 0) {
+        g_direct_signal.store(signal != 0, std::memory_order_release);
+    }
 }
 
 uint64_t xccl_rocm_direct_launch_count(void)
@@ -1031,17 +1228,16 @@ xccl_status_t xccl_rocm_reduce_multi_slots(void *sbuf1, void *sbuf2, void *rbuf,
     // grids), or a one-lane kernel queued behind it (cheaper from a few thousand workgroups on).  The
     // second relies on every result store of the reduction being a write-through store: those are in
     // memory when the reduction kernel ends, and stream order starts the one-lane kernel after that.
-    const bool     want_flag = dev_count != nullptr && dev_flag != nullptr && flagged != nullptr;
-    const bool     tail_ok   = want_flag && g_tail_flag.load(std::memory_order_relaxed) != 0;
-    const unsigned counted   = tail_ok ? g_max_counted_grid.load(std::memory_order_relaxed) : kMaxFlaggedGrid;
-    const bool     in_kernel = want_flag && plan.grid <= counted;
-    const int      words     = in_kernel ? arm_completion(plan, dev_count, dev_flag, flag_words, seq) : 0;
+    const bool want_flag = dev_count != nullptr && dev_flag != nullptr && flagged != nullptr;
+    const int  route     = completion_route(plan, flag_words, false, want_flag, false);
+    const bool in_kernel = route == XCCL_ROCM_ROUTE_SLOTS || route == XCCL_ROCM_ROUTE_COUNTED;
+    const int  words     = in_kernel ? arm_completion(plan, route, dev_count, dev_flag, seq) : 0;
     void *argv[1] = {&plan.args};
     HIP_OR_FAIL(hipLaunchKernel(plan.fn, dim3(plan.grid, 1, 1), dim3(kBlock, 1, 1), argv, plan.lds_bytes,
                                 (hipStream_t)hip_stream));
     if (in_kernel) {
         *flagged = words;
-    } else if (tail_ok) {
+    } else if (route == XCCL_ROCM_ROUTE_TAIL) {
         hipLaunchKernelGGL(tail_flag_kernel, dim3(1), dim3(1), 0, (hipStream_t)hip_stream, dev_flag, seq);
         if (hipGetLastError() == hipSuccess) {
             *flagged = 1; // otherwise the caller waits for the stream, which still works
@@ -1060,8 +1256,14 @@ xccl_status_t xccl_rocm_reduce_multi_flagged_static(void *sbuf1, void *sbuf2, vo
     Plan          plan;
     bool          nothing = false;
     xccl_status_t st      = prepare(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan, &nothing);
-    if (st != XCCL_OK || nothing) {
+    if (st != XCCL_OK) {
         return st;
+    }
+    if (nothing) {
+        // nothing to reduce, but the caller polls the word: a one-lane kernel stores it, in stream order
+        hipLaunchKernelGGL(tail_flag_kernel, dim3(1), dim3(1), 0, (hipStream_t)hip_stream, dev_flag, seq);
+        HIP_OR_FAIL(hipGetLastError());
+        return XCCL_OK;
     }
     if (plan.grid > kMaxFlaggedGrid) {
         fprintf(stderr,
@@ -1190,6 +1392,32 @@ xccl_status_t xccl_rocm_reduce_multi_plan(void *sbuf1, void *sbuf2, void *rbuf, 
     if (name && name_len > 0) {
         const char *n = hipKernelNameRefByPtr(plan.fn, nullptr);
         snprintf(name, name_len, "%s", n ? n : "");
+    }
+    return XCCL_OK;
+}
+
+xccl_status_t xccl_rocm_reduce_multi_route(void *sbuf1, void *sbuf2, void *rbuf, size_t count, size_t size,
+                                           size_t stride, xccl_dt_t dtype, xccl_op_t op, int own_queue,
+                                           unsigned *grid, unsigned *lds_bytes, int *burst, int *route)
+{
+    Plan          plan;
+    xccl_status_t st = make_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, &plan);
+    if (st != XCCL_OK) {
+        return st;
+    }
+    (void)direct_enabled(); // the own queues' environment
+    const KernelEntry *e = lookup(dtype, op);
+    if (grid) {
+        *grid = plan.grid;
+    }
+    if (lds_bytes) {
+        *lds_bytes = plan.lds_bytes;
+    }
+    if (burst) {
+        *burst = plan.fn == e->fn_burst;
+    }
+    if (route) {
+        *route = completion_route(plan, XCCL_ROCM_FLAG_WORDS, own_queue != 0, true, true);
     }
     return XCCL_OK;
 }

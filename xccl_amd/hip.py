@@ -61,6 +61,13 @@ def free(ptr: int):
     check(lib().hipFree(ctypes.c_void_p(ptr)), "hipFree")
 
 
+def malloc_managed(nbytes: int) -> int:
+    """Managed (unified) memory, attached globally."""
+    p = ctypes.c_void_p()
+    check(lib().hipMallocManaged(ctypes.byref(p), ctypes.c_size_t(nbytes), ctypes.c_uint(1)), "hipMallocManaged")
+    return p.value
+
+
 def host_malloc(nbytes: int) -> int:
     p = ctypes.c_void_p()
     check(lib().hipHostMalloc(ctypes.byref(p), ctypes.c_size_t(nbytes), ctypes.c_uint(0)), "hipHostMalloc")
@@ -89,6 +96,16 @@ def memcpy_dtoh(arr: np.ndarray, dptr: int):
     assert arr.flags["C_CONTIGUOUS"]
     check(lib().hipMemcpy(ctypes.c_void_p(arr.ctypes.data), ctypes.c_void_p(dptr), ctypes.c_size_t(arr.nbytes),
                           ctypes.c_int(hipMemcpyDeviceToHost)), "hipMemcpy D2H")
+
+
+def memcpy_raw(dst: int, src: int, nbytes: int, kind: int, stream=None):
+    """hipMemcpy between two addresses; with `stream`, hipMemcpyAsync on it."""
+    if stream is None:
+        check(lib().hipMemcpy(ctypes.c_void_p(dst), ctypes.c_void_p(src), ctypes.c_size_t(nbytes), ctypes.c_int(kind)),
+              "hipMemcpy")
+    else:
+        check(lib().hipMemcpyAsync(ctypes.c_void_p(dst), ctypes.c_void_p(src), ctypes.c_size_t(nbytes), ctypes.c_int(kind),
+                                   ctypes.c_void_p(stream)), "hipMemcpyAsync")
 
 
 def memcpy_dtod(dst: int, src: int, nbytes: int):

@@ -101,6 +101,13 @@ def component_lib():
         lib.xccl_rocm_direct_launch_count.restype = _c.c_uint64
         lib.xccl_rocm_set_direct_queue.argtypes = [_int]
         lib.xccl_rocm_set_direct_queue.restype = None
+        lib.xccl_rocm_reduce_multi_route.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _int,
+                                                     _c.POINTER(_c.c_uint), _c.POINTER(_c.c_uint), _c.POINTER(_int),
+                                                     _c.POINTER(_int)]
+        lib.xccl_rocm_set_counted_grid.argtypes = [_int, _int]
+        lib.xccl_rocm_set_counted_grid.restype = None
+        lib.xccl_rocm_set_direct_options.argtypes = [_int] * 5
+        lib.xccl_rocm_set_direct_options.restype = None
         lib.xccl_rocm_set_slot_max_grid.argtypes = [_int]
         lib.xccl_rocm_set_slot_max_grid.restype = None
         lib.xccl_rocm_reduce_multi_slots.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp, _vp, _vp,
@@ -363,6 +370,21 @@ def reduce_multi_plan(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op):
     if _st(st) != Status.OK:
         raise RuntimeError("xccl_rocm_reduce_multi_plan: %s" % _st(st))
     return {"kernel": name.value.decode(), "grid": grid.value, "block": block.value}
+
+
+ROUTES = ("stream", "slots", "counted", "tail", "signal")     # XCCL_ROCM_ROUTE_*
+
+
+def reduce_multi_route(sbuf1, sbuf2, rbuf, count, size, stride, dtype, op, own_queue=False):
+    """What a launch that reports its own completion would be, on a HIP stream or on the component's own
+    queue: grid, LDS bytes asked for to bound residency, burst kernel or not, completion route."""
+    grid, lds, burst, route = _c.c_uint(0), _c.c_uint(0), _int(0), _int(0)
+    st = component_lib().xccl_rocm_reduce_multi_route(sbuf1, sbuf2, rbuf, count, size, stride, int(dtype), int(op),
+                                                      int(bool(own_queue)), _c.byref(grid), _c.byref(lds),
+                                                      _c.byref(burst), _c.byref(route))
+    if _st(st) != Status.OK:
+        raise RuntimeError("xccl_rocm_reduce_multi_route: %s" % _st(st))
+    return {"grid": grid.value, "lds_bytes": lds.value, "burst": bool(burst.value), "route": ROUTES[route.value]}
 
 
 def bench_region_time_rot(sbuf1, sbuf2, rbuf, rot_count, rot_pitch, count, size, stride, dtype, op, iters: int):
