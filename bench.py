@@ -66,7 +66,7 @@ def parse():
     ap.add_argument("--latency-iters", type=int, default=10000)
     ap.add_argument("--latency-quick", action="store_true", help="3 of the 14 message sizes only")
     ap.add_argument("--profile-mode", nargs="?", const="headline", default=None,
-                    choices=("headline", "config3_int8", "config4_f16", "config4_f64", "small"),
+                    choices=("headline", "footprint", "config3_int8", "config4_f16", "config4_f64", "small"),
                     help="for rocprofv3: only K launches of the named workload (headline: followed by K launches of a "
                          "1 GiB + 1 GiB copy kernel, the known-traffic calibration), nothing else")
     ap.add_argument("--matrix", action="store_true",
@@ -466,24 +466,32 @@ def replay_bench(mc, hip, out_dir):
 def profile_mode(a, mc, hip):
     """Only the launches rocprofv3 is meant to see."""
     from xccl_amd.types import Dt, MemType, Op, Status, dt_size
-    work = {"headline": (Dt.FLOAT32, Op.SUM, 8, SIZE), "config3_int8": (Dt.INT8, Op.PROD, 4, 16777216),
+    work = {"headline": (Dt.FLOAT32, Op.SUM, 8, SIZE), "footprint": (Dt.FLOAT32, Op.SUM, 8, 1 << 28),
+            "config3_int8": (Dt.INT8, Op.PROD, 4, 16777216),
             "config4_f16": (Dt.FLOAT16, Op.SUM, 16, 33554432), "config4_f64": (Dt.FLOAT64, Op.SUM, 16, 33554432),
             "small": (Dt.FLOAT32, Op.SUM, 4, 256)}[a.profile_mode]
     dt, op, nsrc, size = work
     es = dt_size(dt)
     stride = size * es
     slab = Slab(mc, hip)
-    buf = slab.get(dt, nsrc, size, False)
+    # "footprint": 8 x 1 GiB sources, the destination rotating through 4 more vectors (12 GiB touched)
+    rot = 4 if a.profile_mode == "footprint" else 1
+    buf = slab.get(dt, nsrc, size, False, extra=rot)
     stream = mc.component_stream()
     n = a.warmup + a.steps
-    for _ in range(n):
-        st_, _ = mc.xccl_mem_component_reduce_multi_nb(buf, buf + stride, buf + nsrc * stride, nsrc - 1, size, stride,
-                                                       dt, op, MemType.ROCM, None, want_event=False)
+    for i in range(n):
+        st_, _ = mc.xccl_mem_component_reduce_multi_nb(buf, buf + stride, buf + (nsrc + i % rot) * stride, nsrc - 1, size,
+                                                       stride, dt, op, MemType.ROCM, None, want_event=False)
         assert st_ == Status.OK
     hip.stream_synchronize(stream)
     info = {"profile_mode": a.profile_mode, "reduce_launches": n, "dtype": dt.name, "op": op.name, "nsrc": nsrc,
             "size": size, "reduce_algorithmic_bytes": (nsrc + 1) * stride}
     info.update(plan_of(mc, buf, nsrc, size, stride, dt, op))
+    if a.profile_mode == "footprint":
+        for _ in range(n):     # the reduction's reads without its store, same residency bound
+            assert mc.bench_read(buf, stride, nsrc, stride, 10240, stream) == Status.OK
+        hip.stream_synchronize(stream)
+        info.update({"read_only_launches": n, "read_only_bytes": nsrc * stride, "destinations": rot})
     if a.profile_mode == "headline":
         gib = 1 << 30
         for _ in range(n):     # sources 0-3 -> sources 4-7: reads 1 GiB, writes 1 GiB
