@@ -133,9 +133,9 @@ xccl_status_t xccl_rocm_reduce_multi_slots(void *sbuf1, void *sbuf2, void *rbuf,
  * wait for other callers' launches on the same queue; they are not ordered
  * against any HIP stream: issue one only when everything it depends on is
  * complete, and wait for its completion before anything depends on it.
- * `kernarg`: XCCL_ROCM_KERNARG_BYTES of pinned host memory that stay the
- * caller's until the launch is complete (NULL: a ring of the queue's own,
- * and the launch is ordered).
+ * `kernarg`: XCCL_ROCM_KERNARG_BYTES of pinned host memory, or of
+ * xccl_rocm_direct_kernarg_arena, that stay the caller's until the launch is
+ * complete (NULL: a ring of the queue's own, and the launch is ordered).
  * `*flagged` > 0: launched, complete when the first `*flagged` words at
  * `dev_flag` hold `seq`.  `*flagged` == -1: launched, too large to count its
  * own workgroups (more than 6144; XCCL_MC_ROCM_MAX_COUNTED_GRID): complete when
@@ -160,6 +160,18 @@ xccl_status_t xccl_rocm_reduce_multi_direct(void *sbuf1, void *sbuf2, void *rbuf
                                             uint32_t seq, uint64_t *signal,
                                             void *kernarg, int blocking,
                                             int *flagged);
+
+/* `bytes` of DEVICE memory on the current device that the host can write
+ * through the PCIe aperture, for the `kernarg` blocks of
+ * xccl_rocm_reduce_multi_direct: a launch whose arguments sit there starts
+ * 0.8 us sooner than one whose waves fetch them from pinned host memory (an
+ * empty kernel's completion word is seen 3.7 us after the doorbell instead of
+ * 4.55).  One arena per device, allocated on the first call and kept until
+ * the process ends (later calls return the same memory if it is large enough);
+ * NULL where the device's memory is not host-accessible, the own queues are
+ * off or could not be set up, or XCCL_MC_ROCM_DEVICE_KERNARG=0: the caller
+ * then brings pinned host memory. */
+void *xccl_rocm_direct_kernarg_arena(size_t bytes);
 
 /* Nonzero once the launch that armed `signal` (see above) is complete. */
 int xccl_rocm_direct_signal_done(uint64_t signal);

@@ -204,6 +204,50 @@ def test_thread_slots_and_queue_sharing(rocm, oracle):
         buf.close()
 
 
+KERNARG_PROBE = """
+import ctypes, sys
+sys.path.insert(0, %r)
+import numpy as np
+from xccl_amd import hip, mc
+from xccl_amd.types import Dt, MemType, Op, Status
+hip.set_device(0)
+assert mc.xccl_mem_component_init() == Status.OK
+lib = mc.component_lib()
+lib.xccl_rocm_direct_kernarg_arena.restype = ctypes.c_void_p
+lib.xccl_rocm_direct_kernarg_arena.argtypes = [ctypes.c_size_t]
+rng = np.random.default_rng(3)
+ok = True
+for size in (1, 255, 4096, 100003):
+    a = rng.integers(-1000, 1000, (4, size), dtype=np.int32)
+    buf = hip.DeviceBuffer(5 * size * 4)
+    buf.upload(a)
+    before = lib.xccl_rocm_direct_launch_count()
+    for rep in range(50):
+        assert mc.xccl_mem_component_reduce_multi(buf.ptr, buf.ptr + size * 4, buf.ptr + 4 * size * 4, 3, size, size * 4,
+                                                  Dt.INT32, Op.SUM, MemType.ROCM) == Status.OK
+    ok = ok and lib.xccl_rocm_direct_launch_count() - before == 50
+    ok = ok and bool((buf.download(np.int32, size, 4 * size * 4) == a.sum(axis=0, dtype=np.int32)).all())
+    buf.close()
+first = lib.xccl_rocm_direct_kernarg_arena(8192)
+print("arena", bool(first), first == lib.xccl_rocm_direct_kernarg_arena(4096), lib.xccl_rocm_direct_kernarg_arena(1 << 20) is None, "ok", ok)
+"""
+
+
+def test_kernel_arguments_in_device_memory_and_in_pinned_memory():
+    """Launches on the own queues read their arguments from device memory that
+    the host writes through the PCIe aperture (one arena per device, the same
+    memory on every request that fits, none for a larger one); with
+    XCCL_MC_ROCM_DEVICE_KERNARG=0 they read them from pinned host memory.  Both
+    ways: 200 blocking calls on the own queue, results as numpy's."""
+    for env, arena in (({}, "True True True"), ({"XCCL_MC_ROCM_DEVICE_KERNARG": "0"}, "False True True")):
+        e = dict(os.environ)
+        e.pop("XCCL_MC_ROCM_DEVICE_KERNARG", None)
+        e.update(env)
+        out = subprocess.run([sys.executable, "-c", KERNARG_PROBE % ROOT], env=e, capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stdout + out.stderr
+        assert "arena %s ok True" % arena in out.stdout, (env, out.stdout + out.stderr)
+
+
 ROUTE_PROBE = """
 import json, sys
 sys.path.insert(0, %r)

@@ -117,7 +117,8 @@ typedef struct mc_rocm_device {
     int                     *gate_words;  /* pinned, mapped */
     uint32_t                *flag_words; /* pinned, mapped: completion words of the events */
     uint32_t                *arrival_counts; /* device */
-    char                    *kernargs;       /* pinned: XCCL_ROCM_KERNARG_BYTES per event */
+    char                    *kernargs;       /* XCCL_ROCM_KERNARG_BYTES per event: device memory the host can write, else pinned */
+    int                      kernargs_pinned; /* 1: ours to free */
     /* Launches put on each reduction stream, and the highest of them known to be complete (the stream runs
      * them in order).  While the two differ, the stream may hold work nobody has waited for, and a call of that
      * slot stays on the stream, behind it, instead of taking the component's own dispatch queue. */
@@ -227,7 +228,7 @@ static void mc_rocm_device_destroy(mc_rocm_device_t *d)
     if (d->arrival_counts != NULL) {
         (void)hipFree(d->arrival_counts);
     }
-    if (d->kernargs != NULL) {
+    if (d->kernargs != NULL && d->kernargs_pinned) {
         (void)hipHostFree(d->kernargs);
     }
     for (i = 0; i < MC_NUM_STREAMS; i++) {
@@ -241,7 +242,8 @@ static void mc_rocm_device_destroy(mc_rocm_device_t *d)
 /* Stream, events and gate words of one device. */
 static xccl_status_t mc_rocm_device_create_parts(mc_rocm_device_t *d)
 {
-    int i;
+    xccl_status_t st;
+    int           i;
 
     MC_HIP(hipStreamCreateWithFlags(&d->stream[0], hipStreamNonBlocking));
     MC_HIP(hipHostMalloc((void **)&d->gate_words,
@@ -264,8 +266,19 @@ static xccl_status_t mc_rocm_device_create_parts(mc_rocm_device_t *d)
     MC_HIP(hipMemsetAsync(d->arrival_counts, 0,
                           XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_DONE_COUNT_BYTES, d->stream[0]));
     MC_HIP(hipStreamSynchronize(d->stream[0]));
-    MC_HIP(hipHostMalloc((void **)&d->kernargs, XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_KERNARG_BYTES, hipHostMallocDefault));
-    memset(d->kernargs, 0, XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_KERNARG_BYTES);
+    /* compute-unit count, static counter array, the first of the component's own dispatch queues -- behind the
+     * stream: a device serves its most recently created queue fastest (0.6 us per dispatch between the newest and
+     * an older one, measured) */
+    st = xccl_rocm_prepare_device();
+    if (st != XCCL_OK) {
+        return st;
+    }
+    d->kernargs = (char *)xccl_rocm_direct_kernarg_arena(XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_KERNARG_BYTES);
+    if (d->kernargs == NULL) {
+        MC_HIP(hipHostMalloc((void **)&d->kernargs, XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_KERNARG_BYTES, hipHostMallocDefault));
+        memset(d->kernargs, 0, XCCL_ROCM_MC_NUM_EVENTS * XCCL_ROCM_KERNARG_BYTES);
+        d->kernargs_pinned = 1;
+    }
     for (i = 0; i < XCCL_ROCM_MC_NUM_EVENTS; i++) {
         mc_rocm_event_t *ev = &d->events[i];
         ev->kernarg = d->kernargs + (size_t)i * XCCL_ROCM_KERNARG_BYTES;
@@ -278,10 +291,7 @@ static xccl_status_t mc_rocm_device_create_parts(mc_rocm_device_t *d)
         ev->flagged   = 0;
         atomic_store(&ev->is_free, MC_SLOT_FREE);
     }
-    /* compute-unit count, static counter array, the first of the component's own dispatch queues -- last,
-     * behind the stream: a device serves its most recently created queue fastest (0.6 us per dispatch between
-     * the newest and an older one, measured) */
-    return xccl_rocm_prepare_device();
+    return XCCL_OK;
 }
 
 /* All or nothing: a device whose set-up failed half-way keeps no resources and
