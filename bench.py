@@ -75,6 +75,9 @@ def parse():
     ap.add_argument("--replay", action="store_true",
                     help="time whole allreduce collectives of the replayed UCX call sites (8 loopback ranks on the one "
                          "GPU): blocking reductions as in the reference vs stream-ordered ones, scratch cached vs not")
+    ap.add_argument("--latency-child", action="store_true",
+                    help="a handful of small-message rows as JSON and nothing else (the default run starts this in a "
+                         "child process whose runtime keeps its queue rings in device memory)")
     ap.add_argument("--out-dir", default=os.path.join(ROOT, "bench_out"), help="where --matrix / --replay write")
     return ap.parse_args()
 
@@ -236,6 +239,51 @@ def mid_sizes(mc, hip):
             "launched_on": where, "completion": route["route"], "grid": route["grid"]}
         mc.xccl_mem_component_free(slab, MemType.ROCM)
     return rows
+
+
+def latency_child(mc, hip, iters):
+    """A few rows of the small-message sweep: blocking entry, 2/4/8 sources, and 1/2/4 calling threads."""
+    from xccl_amd.types import Dt, Op, Status
+    res = {}
+    maxb = 32768
+    buf = hip.DeviceBuffer(10 * maxb)
+    for j in range(9):
+        mc.datagen_fill(buf.ptr + j * maxb, maxb // 4, Dt.FLOAT32, 5, j)
+    hip.device_synchronize()
+    for nsrc, b in ((2, 4), (4, 1024), (8, 1024), (8, 32768)):
+        st, ns = mc.bench_latency("sync", buf.ptr, buf.ptr + maxb, buf.ptr + 9 * maxb, nsrc - 1, b // 4, maxb, Dt.FLOAT32,
+                                  Op.SUM, iters)
+        assert st == Status.OK, st
+        ns = ns[iters // 10:]
+        res["n%d_%dB" % (nsrc, b)] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
+                                      "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
+    tb = hip.DeviceBuffer(8 * 8192)
+    for th in (1, 2, 4):
+        st, ns = mc.bench_latency_mt(th, 8192, tb.ptr, tb.ptr + 1024, tb.ptr + 4096, 3, 256, 1024, Dt.FLOAT32, Op.SUM,
+                                     iters)
+        assert st == Status.OK
+        ns = ns[:, iters // 10:]
+        res["threads%d_n4_1024B" % th] = {"p50": round(float(np.percentile(ns, 50)) / 1e3, 2),
+                                          "p99": round(float(np.percentile(ns, 99)) / 1e3, 2)}
+    tb.close()
+    buf.close()
+    return res
+
+
+def latency_with_runtime_queues_in_device_memory(iters):
+    """The same rows from a child process started with HSA_ALLOCATE_QUEUE_DEV_MEM=1: the HSA runtime then keeps
+    the packet rings of every queue it creates, the component's own included, in device memory, and the packet
+    processor no longer fetches a packet over PCIe.  A process-wide setting of the runtime, read when it
+    initialises: a deployment's choice, not something a plugin can switch on for its host."""
+    import subprocess
+    env = dict(os.environ, HSA_ALLOCATE_QUEUE_DEV_MEM="1")
+    out = subprocess.run([sys.executable, os.path.abspath(__file__), "--latency-child", "--latency-iters", str(iters)],
+                         env=env, capture_output=True, text=True, timeout=300)
+    if out.returncode != 0:
+        return {"error": (out.stderr or out.stdout)[-300:]}
+    res = json.loads(out.stdout.strip().splitlines()[-1])
+    res["setting"] = "HSA_ALLOCATE_QUEUE_DEV_MEM=1 in the environment of a child process; blocking entry, p50 / p99 in us"
+    return res
 
 
 def latency_extras(mc, hip, buf, iters):
@@ -547,6 +595,9 @@ def main():
     assert mc.xccl_mem_component_init() == Status.OK
     assert bool(mc.dispatch_lib().xccl_mem_component_get(int(MemType.ROCM))), "ROCm component not loaded"
 
+    if a.latency_child:
+        print(json.dumps(latency_child(mc, hip, min(a.latency_iters, 4000))))
+        return 0
     if a.matrix:
         return matrix(mc, hip, a.out_dir)
     if a.replay:
@@ -687,6 +738,7 @@ def main():
         lat, lbuf = latency_sweep(mc, hip, a.latency_iters, a.latency_quick)
         lat.update(latency_extras(mc, hip, lbuf, min(a.latency_iters, 4000)))
         lbuf.close()
+        lat["runtime_queue_rings_in_device_memory"] = latency_with_runtime_queues_in_device_memory(min(a.latency_iters, 4000))
         out["latency_us"] = lat
         out["mid_sizes"] = mid_sizes(mc, hip)
 
