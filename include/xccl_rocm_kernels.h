@@ -209,6 +209,13 @@ int xccl_rocm_direct_signal_done(uint64_t signal);
 void xccl_rocm_set_direct_options(int acquire_system, int queues, int share,
                                   int barrier, int signal);
 
+/* 1: a launch too large to count its own workgroups stays on the own queue,
+ * with a one-lane kernel as a second packet behind it that stores the
+ * completion word (`*flagged` == 1 from xccl_rocm_reduce_multi_direct); 0:
+ * it goes to the HIP stream (or completes by signal, above).  Also
+ * XCCL_MC_ROCM_DIRECT_TAIL. */
+void xccl_rocm_set_direct_tail(int on);
+
 /* Launches that went out on the component's own queues so far (all devices). */
 uint64_t xccl_rocm_direct_launch_count(void);
 

@@ -485,12 +485,13 @@ def test_completion_by_one_word_per_workgroup(rocm, oracle):
 
 
 def test_blocking_calls_take_the_components_own_queue(rocm, oracle):
-    """A blocking reduction small enough to carry its completion word goes out
-    on the component's own dispatch queue, not on a HIP stream -- unless the
-    path is switched off, the call is too large, or the calling thread has
-    stream-ordered launches outstanding that the call has to stay behind.
-    The counter of such launches says which way a call went; the result is
-    the oracle's every time."""
+    """A blocking reduction goes out on the component's own dispatch queue, not
+    on a HIP stream -- a small one carrying its completion word, a large one
+    with a one-lane kernel as a second packet behind it -- unless the path is
+    switched off, the large form is switched off and the call is too large, or
+    the calling thread has launches outstanding on its stream that the call
+    has to stay behind.  The counter of such launches says which way a call
+    went; the result is the oracle's every time."""
     lib = rocm.component_lib()
     dt, op, n2 = Dt.FLOAT32, Op.SUM, 3
     small, large = Case(dt, 5000, n2), Case(dt, 3 * 1024 * 1024, n2)
@@ -511,22 +512,39 @@ def test_blocking_calls_take_the_components_own_queue(rocm, oracle):
         blocking(small, "whichever way: earlier tests may have left stream-ordered launches nobody waited for")
         assert blocking(small, "own queue") == 1
         assert blocking(small, "own queue again") == 1
-        assert blocking(large, "12 MiB vectors: the stream") == 0
+        assert blocking(large, "12 MiB vectors: own queue, completion word from a second packet") == 1
+        lib.xccl_rocm_set_direct_tail(0)
+        assert blocking(large, "12 MiB vectors, second packet switched off: the stream") == 0
+        lib.xccl_rocm_set_direct_tail(1)
         lib.xccl_rocm_set_direct_queue(0)
         assert blocking(small, "switched off") == 0
+        assert blocking(large, "switched off") == 0
         lib.xccl_rocm_set_direct_queue(1)
-        # a stream-ordered launch nobody has waited for: the next blocking call stays behind it on the stream
+        # a launch on the thread's stream that nobody has waited for (no event: nothing but the stream can tell when
+        # it is over): the next blocking call stays behind it on the stream
         p1, p2, pr = large.ptrs()
+        hip.memset(pr, 0x11, large.vbytes)
+        hip.device_synchronize()
+        st, ev = rocm.xccl_mem_component_reduce_multi_nb(p1, p2, pr, n2, large.size, large.stride, dt, op, MemType.ROCM,
+                                                         None, want_event=False)
+        assert st == Status.OK and ev is None
+        assert blocking(small, "behind a launch on the stream") == 0
+        assert_same(large.result(), large.expect(oracle, op)[0], dt, op, "the launch on the stream")   # stream order
+        assert blocking(small, "own queue once the stream has been waited for") == 1
+        # a large stream-ordered launch with an event takes the own queue; a blocking call behind it is ordered behind it
+        hip.memset(pr, 0x12, large.vbytes)
+        hip.device_synchronize()
+        before = lib.xccl_rocm_direct_launch_count()
         st, ev = rocm.xccl_mem_component_reduce_multi_nb(p1, p2, pr, n2, large.size, large.stride, dt, op, MemType.ROCM,
                                                          None)
         assert st == Status.OK and ev is not None
-        assert blocking(small, "behind a stream-ordered launch") == 0
-        assert rocm.xccl_mc_event_query(ev) == Status.OK        # stream order: it has completed as well
+        assert blocking(small, "behind a stream-ordered launch on the own queue") == 1
+        assert lib.xccl_rocm_direct_launch_count() - before == 2
+        assert rocm.xccl_mc_event_query(ev) == Status.OK        # queue order: it has completed as well
         assert rocm.xccl_mc_event_free(ev) == Status.OK
         assert_same(large.result(), large.expect(oracle, op)[0], dt, op, "the stream-ordered launch")
-        assert blocking(small, "own queue once the stream has been waited for") == 1
-        # stream-ordered calls with an event take the own queue as well; a large one behind them goes to the
-        # stream after waiting for them on the host, so the order of one thread's calls holds across both
+        # a small stream-ordered call, then a large one WITHOUT an event, which has to go to the stream: it is issued
+        # only after the first has been waited for on the host, so the order of one thread's calls holds across both
         p1, p2, pr = small.ptrs()
         hip.memset(pr, 0x3D, small.vbytes)
         hip.device_synchronize()
@@ -536,15 +554,15 @@ def test_blocking_calls_take_the_components_own_queue(rocm, oracle):
         assert st == Status.OK and ev_small is not None
         assert lib.xccl_rocm_direct_launch_count() - before == 1
         q1, q2, qr = large.ptrs()
-        st, ev_large = rocm.xccl_mem_component_reduce_multi_nb(q1, q2, qr, n2, large.size, large.stride, dt, op,
-                                                               MemType.ROCM, None)
-        assert st == Status.OK and ev_large is not None
-        assert rocm.xccl_mc_event_query(ev_small) == Status.OK      # the large launch was issued only after it
+        st, none = rocm.xccl_mem_component_reduce_multi_nb(q1, q2, qr, n2, large.size, large.stride, dt, op,
+                                                           MemType.ROCM, None, want_event=False)
+        assert st == Status.OK and none is None
+        assert lib.xccl_rocm_direct_launch_count() - before == 1    # the large one went to the stream
+        assert rocm.xccl_mc_event_query(ev_small) == Status.OK      # and was issued only after the small one
         assert_same(small.result(), small.expect(oracle, op)[0], dt, op, "stream-ordered call on the own queue")
-        t0 = time.time()
-        while rocm.xccl_mc_event_query(ev_large) == Status.INPROGRESS:
-            assert time.time() - t0 < 20.0
-        assert rocm.xccl_mc_event_free(ev_small) == Status.OK and rocm.xccl_mc_event_free(ev_large) == Status.OK
+        assert rocm.xccl_mc_event_free(ev_small) == Status.OK
+        assert blocking(small, "behind the launch on the stream") == 0
+        assert_same(large.result(), large.expect(oracle, op)[0], dt, op, "the large launch on the stream")
         assert blocking(small, "own queue: the large launch has been seen complete") == 1
         # 48 stream-ordered calls in place, none waited for until the end: the queue runs them in order
         chain = Case(Dt.INT32, 3000, 1, alias="s1")
@@ -584,6 +602,7 @@ def test_blocking_calls_take_the_components_own_queue(rocm, oracle):
         assert_same(small.result(), small.expect(oracle, op)[0], dt, op, "after 2000 calls")
     finally:
         lib.xccl_rocm_set_direct_queue(1)
+        lib.xccl_rocm_set_direct_tail(1)
         small.close()
         large.close()
 
@@ -791,7 +810,7 @@ def test_component_works_again_after_close():
     """close() releases a device's streams, events, dispatch queues and the
     code loaded for them -- after everything queued there has completed, also
     launches whose event nobody waited for; the next call sets everything up
-    again.  A fresh process: reductions on the own queue and on the stream,
+    again.  A fresh process: small and large reductions on the own queue,
     four unwaited ones, close (through the dispatcher's free_cache), the same
     reductions once more."""
     import os
@@ -832,7 +851,7 @@ def test_component_works_again_after_close():
     ) % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stdout + out.stderr
-    expect = "[(0, 1, True), (0, 1, True), (0, 0, True)]"
+    expect = "[(0, 1, True), (0, 1, True), (0, 1, True)]"
     assert "before %s after %s" % (expect, expect) in out.stdout, out.stdout + out.stderr
 
 

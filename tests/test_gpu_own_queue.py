@@ -97,12 +97,14 @@ def test_sources_rewritten_in_place_between_own_queue_calls(rocm, acquire):
 
 
 def test_large_launch_on_the_own_queue_completes_through_its_signal(rocm, oracle):
-    """With the signal option on, a call too large to count its own workgroups
-    stays on the own queue and completes through the packet's completion
-    signal: blocking entry, reduce_multi_nb + event_query, and a small blocking
-    call issued behind an unwaited large one (it is ordered behind it).  Off
-    (the default), the same call goes to the HIP stream."""
+    """With the second-packet completion off and the signal option on, a call
+    too large to count its own workgroups stays on the own queue and completes
+    through the packet's completion signal: blocking entry, reduce_multi_nb +
+    event_query, and a small blocking call issued behind an unwaited large one
+    (it is ordered behind it).  With both off, the same call goes to the HIP
+    stream."""
     lib = rocm.component_lib()
+    lib.xccl_rocm_set_direct_tail(0)
     dt, op, n2 = Dt.FLOAT32, Op.SUM, 3
     large, small = Case(dt, 3 * 1024 * 1024 + 5, n2), Case(dt, 3001, 1, alias="s1")
     try:
@@ -111,6 +113,9 @@ def test_large_launch_on_the_own_queue_completes_through_its_signal(rocm, oracle
         want = large.expect(oracle, op)[0]
         p1, p2, pr = large.ptrs()
         assert rocm.reduce_multi_route(p1, p2, pr, n2, large.size, large.stride, dt, op, own_queue=True)["route"] == "stream"
+        lib.xccl_rocm_set_direct_tail(1)
+        assert rocm.reduce_multi_route(p1, p2, pr, n2, large.size, large.stride, dt, op, own_queue=True)["route"] == "tail"
+        lib.xccl_rocm_set_direct_tail(0)
         assert rocm.xccl_mem_component_reduce_multi(p1, p2, pr, n2, large.size, large.stride, dt, op,
                                                     MemType.ROCM) == Status.OK     # leaves the stream idle
         lib.xccl_rocm_set_direct_options(-1, -1, -1, -1, 1)
@@ -160,8 +165,66 @@ def test_large_launch_on_the_own_queue_completes_through_its_signal(rocm, oracle
         assert lib.xccl_rocm_direct_launch_count() - before == 0
     finally:
         lib.xccl_rocm_set_direct_options(-1, -1, -1, -1, 0)
+        lib.xccl_rocm_set_direct_tail(1)
         large.close()
         small.close()
+
+
+@pytest.mark.parametrize("nsrc", [2, 4, 9])
+def test_large_launch_on_the_own_queue_with_a_second_packet(rocm, oracle, nsrc):
+    """The default for calls beyond 64 workgroups: the reduction as one packet,
+    a one-lane kernel that stores the completion word as a second one behind
+    it.  Blocking entry and reduce_multi_nb + event_query over sizes either
+    side of every bound (64 / 65 workgroups, the burst kernel's 2048, ragged
+    tiles, 12 MiB vectors), in place, and 40 events in flight at once."""
+    lib = rocm.component_lib()
+    dt, op, n2 = Dt.INT32, Op.SUM, nsrc - 1
+    for size in (64 * 256, 64 * 256 + 1, 65 * 256 - 3, 2048 * 256, 2049 * 256 + 7, 3 * 1024 * 1024 + 5):
+        c = Case(dt, size, n2, alias="s1" if size % 2 else None)
+        try:
+            c.fill_random(oracle, 500 + nsrc)
+            c.upload()
+            p1, p2, pr = c.ptrs()
+            want, _ = c.expect(oracle, op)
+            route = rocm.reduce_multi_route(p1, p2, pr, n2, size, c.stride, dt, op, own_queue=True)
+            assert route["route"] == ("counted" if route["grid"] <= 64 else "tail"), (size, route)
+            before = lib.xccl_rocm_direct_launch_count()
+            assert rocm.xccl_mem_component_reduce_multi(p1, p2, pr, n2, size, c.stride, dt, op, MemType.ROCM) == Status.OK
+            assert lib.xccl_rocm_direct_launch_count() - before == 1
+            assert_same(c.result(), want, dt, op, "blocking, %d elements" % size)
+            c.upload()
+            st, ev = rocm.xccl_mem_component_reduce_multi_nb(p1, p2, pr, n2, size, c.stride, dt, op, MemType.ROCM, None)
+            assert st == Status.OK and ev is not None
+            t0 = time.time()
+            while rocm.xccl_mc_event_query(ev) == Status.INPROGRESS:
+                assert time.time() - t0 < 20.0
+            assert rocm.xccl_mc_event_query(ev) == Status.OK and rocm.xccl_mc_event_free(ev) == Status.OK
+            assert_same(c.result(), want, dt, op, "stream-ordered, %d elements" % size)
+        finally:
+            c.close()
+    # 40 stream-ordered launches of 300 workgroups in place, none waited for until the end: 80 packets in order
+    chain = Case(dt, 300 * 256, 1, alias="s1")
+    try:
+        chain.fill_random(oracle, 600 + nsrc)
+        chain.upload()
+        c1, c2, cr = chain.ptrs()
+        evs = []
+        for rep in range(40):
+            st, e = rocm.xccl_mem_component_reduce_multi_nb(c1, c2, cr, 1, chain.size, chain.stride, dt, op, MemType.ROCM,
+                                                            None)
+            assert st == Status.OK and e is not None
+            evs.append(e)
+        t0 = time.time()
+        while rocm.xccl_mc_event_query(evs[-1]) == Status.INPROGRESS:
+            assert time.time() - t0 < 20.0
+        for e in evs:
+            assert rocm.xccl_mc_event_query(e) == Status.OK and rocm.xccl_mc_event_free(e) == Status.OK
+        a = chain.host[chain.o1: chain.o1 + chain.vbytes].view(np.int32).astype(np.int64)
+        b = chain.host[chain.o2: chain.o2 + chain.vbytes].view(np.int32).astype(np.int64)
+        want = ((a + 40 * b) & 0xffffffff).astype(np.uint32).view(np.int32)
+        assert chain.result().view(np.int32).tolist() == want.tolist()
+    finally:
+        chain.close()
 
 
 def test_thread_slots_and_queue_sharing(rocm, oracle):
@@ -282,15 +345,20 @@ def test_every_launch_shape_variable_changes_the_route_it_names():
     fresh process, changes exactly what it names in the plan of a call."""
     d = _routes({})
     assert d["four_tiles_stream"] == {"grid": 4, "lds_bytes": 0, "burst": True, "route": "slots"}
-    assert d["small_4src_own"] == {"grid": 1000, "lds_bytes": 0, "burst": True, "route": "counted"}
-    assert d["mid_stream"]["route"] == "tail" and d["mid_own"]["route"] == "counted" and not d["mid_own"]["burst"]
-    assert d["large_stream"]["route"] == "tail" and d["large_own"]["route"] == "stream"
+    assert d["four_tiles_own"]["route"] == "slots"
+    assert d["small_4src_own"] == {"grid": 1000, "lds_bytes": 0, "burst": True, "route": "tail"}
+    assert d["mid_stream"]["route"] == "tail" and d["mid_own"]["route"] == "tail" and not d["mid_own"]["burst"]
+    assert d["large_stream"]["route"] == "tail" and d["large_own"]["route"] == "tail" and d["huge_own"]["route"] == "tail"
+    n = _routes({"XCCL_MC_ROCM_DIRECT_TAIL": "0"})
+    assert n["small_4src_own"]["route"] == "counted" and n["mid_own"]["route"] == "counted"     # up to 6144 workgroups
+    assert n["large_own"]["route"] == "stream" and n["large_stream"] == d["large_stream"]
     assert d["huge_stream"] == {"grid": 262144, "lds_bytes": 10752, "burst": False, "route": "tail"}   # 15 resident per CU
     assert d["mid_stream"]["lds_bytes"] == 0           # 9 x 4 MiB: fits the memory-side cache, no residency bound
 
     c = _routes({"XCCL_MC_ROCM_MAX_COUNTED_GRID": "5000"})
     assert c["mid_stream"]["route"] == "counted" and c["mid_own"]["route"] == "counted" and c["large_stream"]["route"] == "tail"
-    c = _routes({"XCCL_MC_ROCM_MAX_COUNTED_GRID": "512"})
+    assert c["large_own"]["route"] == "tail"
+    c = _routes({"XCCL_MC_ROCM_MAX_COUNTED_GRID": "512", "XCCL_MC_ROCM_DIRECT_TAIL": "0"})
     assert c["small_4src_stream"]["route"] == "tail" and c["small_4src_own"]["route"] == "stream"
     assert c["four_tiles_own"]["route"] == "slots"
     t = _routes({"XCCL_MC_ROCM_TAIL_FLAG": "0"})
@@ -304,7 +372,7 @@ def test_every_launch_shape_variable_changes_the_route_it_names():
     b = _routes({"XCCL_MC_ROCM_BLOCKS_PER_CU": "4"})
     cap = b["huge_stream"]["grid"]                      # 4 x the device's compute units
     assert cap % 4 == 0 and 4 <= cap < 4096 and b["large_stream"]["grid"] == cap and b["mid_stream"]["grid"] == cap
-    assert b["small_4src_stream"]["grid"] == 1000 and b["mid_own"]["route"] == "counted"
+    assert b["small_4src_stream"]["grid"] == 1000 and b["mid_own"]["route"] == "tail"
     assert _routes({"XCCL_MC_ROCM_BLOCKS_PER_CU": "8"})["huge_stream"]["grid"] == 2 * cap
     u = _routes({"XCCL_MC_ROCM_BURST_MAX_GRID": "0"})
     assert not u["four_tiles_stream"]["burst"] and not u["small_4src_own"]["burst"]
@@ -312,6 +380,7 @@ def test_every_launch_shape_variable_changes_the_route_it_names():
     assert u["mid_own"]["burst"] and not u["large_own"]["burst"]
     s = _routes({"XCCL_MC_ROCM_SLOT_MAX_GRID": "0"})
     assert s["four_tiles_stream"]["route"] == "counted" and s["four_tiles_own"]["route"] == "counted"
-    g = _routes({"XCCL_MC_ROCM_DIRECT_SIGNAL": "1"})
+    g = _routes({"XCCL_MC_ROCM_DIRECT_SIGNAL": "1", "XCCL_MC_ROCM_DIRECT_TAIL": "0"})
     assert g["large_own"]["route"] == "signal" and g["huge_own"]["route"] == "signal" and g["mid_own"]["route"] == "counted"
     assert g["large_stream"] == d["large_stream"]
+    assert _routes({"XCCL_MC_ROCM_DIRECT_SIGNAL": "1"})["large_own"]["route"] == "tail"         # the second packet comes first

@@ -88,6 +88,7 @@ struct DirectDevice {
     // arguments sit there starts 0.8 us sooner than one whose waves fetch them from pinned host memory (an
     // empty kernel's completion word is seen 3.7 us after the doorbell instead of 4.55).  Allocated once per
     // device and kept until the process ends, whatever happens to the queues.
+    DirectKernel                                  tail_kernel{}; // xccl_rocm_tail_flag_kernel, looked up on first use
     void                                         *arena       = nullptr;
     size_t                                        arena_bytes = 0;
     bool                                          arena_tried = false;
@@ -113,6 +114,9 @@ std::atomic<int>      g_direct_queues{kDefaultDirectQueues};
 std::atomic<int>      g_direct_share{1};
 std::atomic<int>      g_direct_barrier{0};
 std::atomic<int>      g_direct_signal{0};
+//   g_direct_tail     1: such launches stay on the own queue with a one-lane kernel as a second packet behind
+//                     them that stores the completion word (XCCL_MC_ROCM_DIRECT_TAIL)
+std::atomic<int>      g_direct_tail{1};
 
 bool direct_enabled()
 {
@@ -124,6 +128,10 @@ bool direct_enabled()
         const char *h = getenv("XCCL_MC_ROCM_DIRECT_SHARE");
         const char *b = getenv("XCCL_MC_ROCM_DIRECT_BARRIER");
         const char *g = getenv("XCCL_MC_ROCM_DIRECT_SIGNAL");
+        const char *t = getenv("XCCL_MC_ROCM_DIRECT_TAIL");
+        if (t != nullptr) {
+            g_direct_tail.store(atoi(t) != 0, std::memory_order_release);
+        }
         if (a != nullptr) {
             g_direct_acquire.store(strcmp(a, "system") == 0 ? HSA_FENCE_SCOPE_SYSTEM : HSA_FENCE_SCOPE_AGENT,
                                    std::memory_order_release);
@@ -156,6 +164,13 @@ bool direct_enabled()
                     m_ ? m_ : "unknown status");                                                           \
             return false;                                                                                  \
         }                                                                                                  \
+    } while (0)
+
+#define HSA_OR_GIVE_UP_STATUS(call)            \
+    do {                                       \
+        if ((call) != HSA_STATUS_SUCCESS) {    \
+            return XCCL_ERR_NO_RESOURCE;       \
+        }                                      \
     } while (0)
 
 struct AgentSearch {
@@ -501,6 +516,72 @@ xccl_status_t direct_launch(DirectDevice &dd, int slot, const Plan &plan, uint64
     return XCCL_OK;
 }
 
+// The one-lane kernel that stores `seq` to `flag`, as a packet with the barrier
+// bit on queue `slot`; `kernarg`: 16 bytes the caller keeps until it has run.
+xccl_status_t direct_launch_tail(DirectDevice &dd, int slot, uint32_t *flag, uint32_t seq, void *kernarg)
+{
+    DirectQueue *dq = nullptr;
+    if (slot < 0 || slot >= kMaxDirectQueues || kernarg == nullptr || !direct_queue(dd, slot, &dq)) {
+        return XCCL_ERR_NO_RESOURCE;
+    }
+    if (dd.tail_kernel.object == 0) {
+        std::lock_guard<std::mutex> guard(dd.lock);
+        if (dd.tail_kernel.object == 0) {
+            hsa_executable_symbol_t sym;
+            uint32_t                kernarg_bytes = 0, priv = 0;
+            DirectKernel            k;
+            HSA_OR_GIVE_UP_STATUS(hsa_executable_get_symbol_by_name(dd.exe, "xccl_rocm_tail_flag_kernel.kd", &dd.agent, &sym));
+            HSA_OR_GIVE_UP_STATUS(hsa_executable_symbol_get_info(sym, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_OBJECT, &k.object));
+            HSA_OR_GIVE_UP_STATUS(hsa_executable_symbol_get_info(sym, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_KERNARG_SEGMENT_SIZE, &kernarg_bytes));
+            HSA_OR_GIVE_UP_STATUS(hsa_executable_symbol_get_info(sym, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_GROUP_SEGMENT_SIZE, &k.group));
+            HSA_OR_GIVE_UP_STATUS(hsa_executable_symbol_get_info(sym, HSA_EXECUTABLE_SYMBOL_INFO_KERNEL_PRIVATE_SEGMENT_SIZE, &priv));
+            if (kernarg_bytes > 16 || priv != 0 || k.object == 0) {
+                return XCCL_ERR_NO_RESOURCE;
+            }
+            dd.tail_kernel = k;
+        }
+    }
+    struct {
+        uint32_t *flag;
+        uint32_t  seq, pad;
+    } args = {flag, seq, 0};
+    memcpy(kernarg, &args, sizeof(args));
+#if defined(__x86_64__) || defined(__i386__)
+    _mm_sfence();
+#else
+    __atomic_thread_fence(__ATOMIC_SEQ_CST);
+#endif
+    hsa_queue_t   *q   = dq->q;
+    const uint64_t idx = hsa_queue_add_write_index_scacq_screl(q, 1);
+    while (idx - hsa_queue_load_read_index_scacquire(q) >= q->size) {
+        if (g_direct_failed.load(std::memory_order_acquire) != 0) {
+            return XCCL_ERR_NO_RESOURCE;
+        }
+    }
+    hsa_kernel_dispatch_packet_t *p = static_cast<hsa_kernel_dispatch_packet_t *>(q->base_address) + (idx & (q->size - 1));
+    p->workgroup_size_x     = 1;
+    p->workgroup_size_y     = 1;
+    p->workgroup_size_z     = 1;
+    p->reserved0            = 0;
+    p->grid_size_x          = 1;
+    p->grid_size_y          = 1;
+    p->grid_size_z          = 1;
+    p->private_segment_size = 0;
+    p->group_segment_size   = dd.tail_kernel.group;
+    p->kernel_object        = dd.tail_kernel.object;
+    p->kernarg_address      = kernarg;
+    p->reserved2            = 0;
+    p->completion_signal.handle = 0;
+    const uint32_t header = (uint32_t)HSA_PACKET_TYPE_KERNEL_DISPATCH << HSA_PACKET_HEADER_TYPE |
+                            1u << HSA_PACKET_HEADER_BARRIER |
+                            (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE |
+                            (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE;
+    const uint32_t setup  = 1u << HSA_KERNEL_DISPATCH_PACKET_SETUP_DIMENSIONS;
+    __atomic_store_n(reinterpret_cast<uint32_t *>(p), header | setup << 16, __ATOMIC_RELEASE);
+    hsa_signal_store_screlease(q->doorbell_signal, (hsa_signal_value_t)idx);
+    return XCCL_OK;
+}
+
 // Waits until everything queued on `q` has completed: a barrier packet with a
 // completion signal goes in behind it (a stream-ordered launch whose event
 // nobody waited for may still be queued or running when the component closes).
@@ -562,6 +643,7 @@ void direct_destroy(DirectDevice &dd)
     }
     dd.signals.clear();
     dd.kernels.clear();
+    dd.tail_kernel = DirectKernel{};
     dd.generation.fetch_add(1, std::memory_order_release); // kernel descriptors cached by the threads are stale now
     if (dd.exe.handle != 0) {
         (void)hsa_executable_destroy(dd.exe);
@@ -590,6 +672,11 @@ void direct_read_env()
 bool direct_signal_enabled()
 {
     return g_direct_signal.load(std::memory_order_relaxed) != 0;
+}
+
+bool direct_tail_enabled()
+{
+    return g_direct_tail.load(std::memory_order_relaxed) != 0;
 }
 
 // Loading the code and creating a queue takes milliseconds, which belong into a
@@ -655,6 +742,29 @@ xccl_status_t xccl_rocm_reduce_multi_direct(void *sbuf1, void *sbuf2, void *rbuf
     if (route == XCCL_ROCM_ROUTE_STREAM) {
         return XCCL_OK; // too many workgroups to count themselves: the launch completes through the stream
     }
+    if (route == XCCL_ROCM_ROUTE_TAIL) {
+        // the reduction, then a one-lane kernel behind it that stores the word; its 16 bytes of arguments sit
+        // behind the reduction's in the caller's block
+        if (kernarg == nullptr) {
+            return XCCL_OK;
+        }
+        static_assert(sizeof(ReduceArgs) + 16 <= XCCL_ROCM_KERNARG_BYTES, "room for the tail kernel's arguments");
+        if (direct_launch(*dd, queue_slot, plan, 0, ordered, kernarg) != XCCL_OK) {
+            return XCCL_OK;
+        }
+        if (direct_launch_tail(*dd, queue_slot, dev_flag, seq, static_cast<char *>(kernarg) + XCCL_ROCM_KERNARG_BYTES - 16) !=
+            XCCL_OK) {
+            // the reduction is queued but no kernel will tell when it is over: wait for the queue to drain and
+            // store the word from here (it is host memory, at the same address on both sides)
+            DirectQueue *dq = nullptr;
+            if (direct_queue(*dd, queue_slot, &dq)) {
+                direct_drain(dq->q, 10000000000ull);
+            }
+            __atomic_store_n(dev_flag, seq, __ATOMIC_RELEASE);
+        }
+        *flagged = 1;
+        return XCCL_OK;
+    }
     if (route == XCCL_ROCM_ROUTE_SIGNAL) {
         if (*signal == 0 && !direct_signal_create(*dd, signal)) {
             return XCCL_OK;
@@ -676,6 +786,12 @@ int xccl_rocm_direct_signal_done(uint64_t signal)
 {
     return hsa_signal_load_scacquire(hsa_signal_t{signal}) == 0;
 }
+void xccl_rocm_set_direct_tail(int on)
+{
+    (void)direct_enabled();
+    g_direct_tail.store(on != 0, std::memory_order_release);
+}
+
 void xccl_rocm_set_direct_options(int acquire_system, int queues, int share, int barrier, int signal)
 {
     (void)direct_enabled(); // environment first, so that it does not overwrite these later

@@ -49,6 +49,7 @@ uint64_t clock_ns(); // CLOCK_MONOTONIC
 // direct_queue.hip
 void direct_read_env();            // reads the own queues' environment variables, once
 bool direct_signal_enabled();      // large launches may complete through a packet's completion signal
+bool direct_tail_enabled();        // ... or through a one-lane kernel as a second packet behind them
 void direct_prepare_first_queue(); // loads the kernels' code objects and creates queue 0 of the current device
 
 #define HIP_OR_FAIL(call)                                                                          \

@@ -37,3 +37,13 @@ const KernelEntry *lookup_fp(int kop, int bytes)
 }
 
 } // namespace xccl_rocm
+
+// The completion word of a launch too large to count its own workgroups, as
+// a second packet behind it on the component's own dispatch queue: one lane
+// stores the sequence number once everything queued before has completed
+// (the packet carries the barrier bit).  Lives in this unit because the own
+// queues load their kernels from the five embedded code objects.
+extern "C" __global__ void xccl_rocm_tail_flag_kernel(uint32_t *flag, uint32_t seq)
+{
+    __hip_atomic_store(flag, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}

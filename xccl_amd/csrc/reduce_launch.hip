@@ -31,10 +31,15 @@ std::atomic<int> g_blocks_per_cu{-1}; // -1: not read from the environment yet
 std::atomic<int> g_resident{0};
 std::atomic<int> g_tail_flag{1};
 std::atomic<unsigned> g_shape_epoch{0}; // bumped when a launch-shape knob changes
-// the same bound for launches on the component's own dispatch queue, where the alternative to counting is the
-// stream path as a whole (blocking call, us, counting on the own queue / queued kernel on the stream: 3072
-// workgroups 7.8 / 8.8-9.3, 4096: 8.2 / 8.9-9.4, 6144: 9.2 / 9.2-9.4, 8192: 10.0 / 9.6-9.8)
-std::atomic<unsigned> g_direct_counted_grid{6144};
+// The same bound for launches on the component's own dispatch queue, where a larger launch gets a one-lane kernel
+// as a second packet behind it.  With the kernel arguments in device memory that second packet costs less than the
+// second level of arrival counting (grids beyond 64 workgroups count in two levels): blocking call, us, counting /
+// second packet, 2 | 8 sources: 32 workgroups 5.49 / 5.77 | 5.64 / 5.91, 64: 5.51 / 5.83 | 5.83 / 5.91, 96: 5.83 /
+// 5.83 | 5.99 / 5.87, 256: 5.83 / 5.83 | 6.02 / 5.92, 1024: 6.22 / 5.87 | 6.61 / 6.37, 2048: 6.58 / 6.33 | 7.43 /
+// 6.73, 4096: 7.34 / 6.76 | 9.45 / 9.25, 8192: 8.83 / 7.76 | 16.0 / 15.2.  (With that option off the bound that
+// serves is 6144: counting against the HIP stream's queued kernel.)
+constexpr unsigned kCountedGridUnset = ~0u; // 64 with the second packet, 6144 without
+std::atomic<unsigned> g_direct_counted_grid{kCountedGridUnset};
 std::atomic<unsigned> g_max_counted_grid{2048}; // measured (blocking call, us, counting / queued kernel): 512 workgroups 8.0 / 9.2, 2048: 8.6-9.7 / 9.4-9.5, 8192: 10.4 / 10.0
 // Launches of at most this many workgroups (and at least 4 sources; up to 3 the
 // walk has every load in flight anyway) use the burst kernel: all loads of a
@@ -359,15 +364,20 @@ xccl_status_t prepare(void *s1, void *s2, void *dst, size_t count, size_t size, 
 // How the host learns that a launch is complete (values of XCCL_ROCM_ROUTE_*):
 // one word per workgroup for a handful of workgroups, a word written by the
 // last workgroup to arrive for small grids, and for larger ones a one-lane
-// kernel queued behind the launch on a HIP stream or the packet's completion
-// signal on the component's own queue; else the stream itself.
+// kernel queued behind the launch (on a HIP stream, or as a second packet on
+// the component's own queue) or the packet's completion signal on the own
+// queue; else the stream itself.
 int completion_route(const Plan &plan, uint32_t flag_words, bool own_queue, bool want_flag, bool has_signal)
 {
     if (!want_flag) {
         return XCCL_ROCM_ROUTE_STREAM;
     }
     const bool     tail_ok   = g_tail_flag.load(std::memory_order_relaxed) != 0;
-    const unsigned counted   = own_queue ? g_direct_counted_grid.load(std::memory_order_relaxed)
+    unsigned       own_bound = g_direct_counted_grid.load(std::memory_order_relaxed);
+    if (own_bound == kCountedGridUnset) {
+        own_bound = direct_tail_enabled() ? 64u : 6144u;
+    }
+    const unsigned counted   = own_queue ? own_bound
                                : tail_ok ? g_max_counted_grid.load(std::memory_order_relaxed)
                                          : kMaxFlaggedGrid;
     const unsigned slots_max = flag_words < XCCL_ROCM_FLAG_WORDS ? flag_words : XCCL_ROCM_FLAG_WORDS;
@@ -377,8 +387,10 @@ int completion_route(const Plan &plan, uint32_t flag_words, bool own_queue, bool
         return by_slots ? XCCL_ROCM_ROUTE_SLOTS : XCCL_ROCM_ROUTE_COUNTED;
     }
     if (own_queue) {
-        return has_signal && direct_signal_enabled() ? XCCL_ROCM_ROUTE_SIGNAL
-                                                                                         : XCCL_ROCM_ROUTE_STREAM;
+        if (direct_tail_enabled()) {
+            return XCCL_ROCM_ROUTE_TAIL;
+        }
+        return has_signal && direct_signal_enabled() ? XCCL_ROCM_ROUTE_SIGNAL : XCCL_ROCM_ROUTE_STREAM;
     }
     return tail_ok ? XCCL_ROCM_ROUTE_TAIL : XCCL_ROCM_ROUTE_STREAM;
 }

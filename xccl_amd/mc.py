@@ -106,6 +106,8 @@ def component_lib():
                                                      _c.POINTER(_int)]
         lib.xccl_rocm_set_counted_grid.argtypes = [_int, _int]
         lib.xccl_rocm_set_counted_grid.restype = None
+        lib.xccl_rocm_set_direct_tail.argtypes = [_int]
+        lib.xccl_rocm_set_direct_tail.restype = None
         lib.xccl_rocm_set_direct_options.argtypes = [_int] * 5
         lib.xccl_rocm_set_direct_options.restype = None
         lib.xccl_rocm_set_slot_max_grid.argtypes = [_int]
