@@ -137,17 +137,21 @@ xccl_status_t xccl_rocm_reduce_multi_slots(void *sbuf1, void *sbuf2, void *rbuf,
  * xccl_rocm_direct_kernarg_arena, that stay the caller's until the launch is
  * complete (NULL: a ring of the queue's own, and the launch is ordered).
  * `*flagged` > 0: launched, complete when the first `*flagged` words at
- * `dev_flag` hold `seq`.  `*flagged` == -1: launched, too large to count its
- * own workgroups (more than 6144; XCCL_MC_ROCM_MAX_COUNTED_GRID): complete when
+ * `dev_flag` hold `seq`: written by the launch itself up to 64 workgroups, by
+ * a one-lane kernel that goes out as a second packet behind it beyond
+ * (xccl_rocm_set_direct_tail; needs `kernarg`).  `*flagged` == -1: launched,
+ * too large to count its own workgroups, the second packet switched off and
+ * completion by signal switched on: complete when
  * xccl_rocm_direct_signal_done(*signal) -- `*signal` is created on first need
  * (0 before) and belongs to the queues: it goes with
  * xccl_rocm_direct_queue_destroy.  `*flagged` == 0 with XCCL_OK: nothing was
  * launched and the caller uses xccl_rocm_reduce_multi_slots instead -- the
- * call is too large and `signal` is NULL or that path is off, has size 0, the
- * slot has no queue, the queue could not be set up (said once on stderr), or
- * the path is switched off (XCCL_MC_ROCM_DIRECT_QUEUE=0 or
- * xccl_rocm_set_direct_queue(0)).  Blocking call, 4 sources x 32 KiB: p50
- * 6.7 us against 7.6 us on a HIP stream, p99 7.0 against 11.3 us.  No
+ * call is too large for its own word (more than 6144 workgroups then) and
+ * both of those are off, has size 0, the slot has no queue, the queue could
+ * not be set up (said once on stderr), or the path is switched off
+ * (XCCL_MC_ROCM_DIRECT_QUEUE=0 or xccl_rocm_set_direct_queue(0)).  Blocking
+ * call, 4 sources x 1 KiB: p50 4.6 us against 7.1 us on a HIP stream, p99 4.8
+ * against 10-12 us; 8 sources x 16 MiB: 26.4-26.9 against 28.4-28.8 us.  No
  * counterpart in the reference.
  */
 #define XCCL_ROCM_KERNARG_BYTES 128
@@ -194,7 +198,10 @@ int xccl_rocm_direct_signal_done(uint64_t signal);
  *                   on these queues and complete through a completion signal;
  *                   0 (default): they go to the HIP stream
  *                   (XCCL_MC_ROCM_DIRECT_SIGNAL)
- * Measured, blocking call, 4 sources x 1 KiB, p50 / p99 in us, 1 / 2 / 4
+ * Measured with the kernel arguments still in pinned host memory (in device
+ * memory every row is 0.8 us lower and the shipped setting gives 4.6 / 4.8,
+ * 5.3-5.5 / 5.7-6.0, 5.5-5.9 / 6.2-6.5), blocking call, 4 sources x 1 KiB,
+ * p50 / p99 in us, 1 / 2 / 4
  * calling threads: two queues shared, no barrier 5.5 / 5.8, 6.3 / 8.7,
  * 6.7-7.2 / 13.2; shared, with barrier 6.3 / 7.1, 6.1-6.4 / 8.8, 6.9-7.7 /
  * 13.6; two queues not shared (threads 3 and 4 on HIP streams) 5.4 / 5.8,
@@ -209,11 +216,14 @@ int xccl_rocm_direct_signal_done(uint64_t signal);
 void xccl_rocm_set_direct_options(int acquire_system, int queues, int share,
                                   int barrier, int signal);
 
-/* 1: a launch too large to count its own workgroups stays on the own queue,
- * with a one-lane kernel as a second packet behind it that stores the
- * completion word (`*flagged` == 1 from xccl_rocm_reduce_multi_direct); 0:
- * it goes to the HIP stream (or completes by signal, above).  Also
- * XCCL_MC_ROCM_DIRECT_TAIL. */
+/* 1 (default): a launch too large to count its own workgroups stays on the
+ * own queue, with a one-lane kernel as a second packet behind it that stores
+ * the completion word (`*flagged` == 1 from xccl_rocm_reduce_multi_direct);
+ * 0: it goes to the HIP stream (or completes by signal, above).  Also
+ * XCCL_MC_ROCM_DIRECT_TAIL.  Blocking call, us, this / HIP stream with a
+ * queued one-lane kernel / completion signal, 8 sources x 8 MiB 15.4 / 17.3 /
+ * 16.6, x 16 MiB 26.4 / 28.8 / 27.7, x 64 MiB 93.5 / 95.8 / 94.6, x 256 MiB
+ * 353.7 / 357.8 / 355.2; 2 sources x 8 MiB 7.7 / 9.7 / 8.8. */
 void xccl_rocm_set_direct_tail(int on);
 
 /* Launches that went out on the component's own queues so far (all devices). */
@@ -311,7 +321,8 @@ void xccl_rocm_set_slot_max_grid(int max_grid);
 
 /* Largest launch, in workgroups, that counts its own arrivals for the
  * completion word: on a HIP stream (default 2048; larger ones get a one-lane
- * kernel queued behind them) and on the component's own queue (default 6144).
+ * kernel queued behind them) and on the component's own queue (default 64;
+ * 6144 with the second packet of xccl_rocm_set_direct_tail switched off).
  * Negative = leave alone.  Also XCCL_MC_ROCM_MAX_COUNTED_GRID (sets both).
  * For measurement and tests. */
 void xccl_rocm_set_counted_grid(int on_stream, int on_own_queue);

@@ -103,19 +103,18 @@ extern "C" {
  *                    (the one the synchronous entries use on that thread), so
  *                    successive calls of one thread are ordered among
  *                    themselves.  That queue is a HIP stream (get_stream) for
- *                    calls without an event and for large ones; a call that
- *                    has an event and is small enough to report its own
- *                    completion goes out on a dispatch queue of the
- *                    component's own instead when the stream holds nothing
- *                    it would have to stay behind (5.2-6.6 us per call instead
- *                    of 7.0-7.9; XCCL_MC_ROCM_DIRECT_QUEUE=0 switches that
- *                    off).  The order of one thread's calls holds across the
- *                    two; only the event tells when such a call is complete.  Threads are spread round-robin over up to 4
- *                    streams per device (XCCL_MC_ROCM_THREAD_STREAMS, 1..4),
- *                    so that blocking calls of several threads
- *                    (XCCL_THREAD_MODE_MULTIPLE) do not queue up behind each
- *                    other's kernels; calls of different threads are not
- *                    ordered among themselves;
+ *                    calls without an event; a call that has an event goes out
+ *                    on a dispatch queue of the component's own instead when
+ *                    the stream holds nothing it would have to stay behind
+ *                    (4.4-5.6 us per small call instead of 6.8-7.7;
+ *                    XCCL_MC_ROCM_DIRECT_QUEUE=0 switches that off).  The
+ *                    order of one thread's calls holds across the two; only
+ *                    the event tells when such a call is complete.  Threads
+ *                    are spread round-robin over up to 4 streams per device
+ *                    (XCCL_MC_ROCM_THREAD_STREAMS, 1..4), so that blocking
+ *                    calls of several threads (XCCL_THREAD_MODE_MULTIPLE) do
+ *                    not queue up behind each other's kernels; calls of
+ *                    different threads are not ordered among themselves;
  *   stream != NULL : enqueue on *(hipStream_t*)stream->stream.
  *   event  != NULL : *event receives a pooled event recorded right after the
  *                    kernel; poll it with event_query (XCCL_INPROGRESS /
