@@ -39,7 +39,9 @@ namespace {
 // threads' launches on the same queue.
 //   Two queues per device by default, shared by the component's four thread
 // slots (slot s uses queue s mod 2), each created when a thread that uses it
-// first calls, behind that slot's HIP stream.  Measured, blocking call, 4
+// first calls, behind that slot's HIP stream.  Measured with the argument
+// blocks in pinned host memory (in device memory every figure is 0.7-1 us
+// lower, and four threads see 5.5-5.9 / 6.2-6.5), blocking call, 4
 // sources x 1 KiB, p50 / p99 in us, 1 / 2 / 4 calling threads: this 5.5 / 5.8,
 // 6.3 / 8.7, 6.7-7.2 / 13.2; with the barrier bit on every packet 6.3 / 7.1,
 // 6.1-6.4 / 8.8, 6.9-7.7 / 13.6; slots 2 and 3 on HIP streams instead 5.4 / 5.8,
@@ -84,11 +86,11 @@ struct DirectDevice {
     std::unordered_map<const void *, DirectKernel> kernels; // by HIP function pointer
     DirectQueue                                   queue[kMaxDirectQueues];
     std::vector<hsa_signal_t>                     signals; // completion signals handed out, destroyed with the queues
+    DirectKernel                                  tail_kernel{}; // xccl_rocm_tail_flag_kernel, looked up on first use
     // Kernel-argument blocks in DEVICE memory that the host writes through the PCIe aperture: a launch whose
     // arguments sit there starts 0.8 us sooner than one whose waves fetch them from pinned host memory (an
     // empty kernel's completion word is seen 3.7 us after the doorbell instead of 4.55).  Allocated once per
     // device and kept until the process ends, whatever happens to the queues.
-    DirectKernel                                  tail_kernel{}; // xccl_rocm_tail_flag_kernel, looked up on first use
     void                                         *arena       = nullptr;
     size_t                                        arena_bytes = 0;
     bool                                          arena_tried = false;
@@ -524,7 +526,7 @@ xccl_status_t direct_launch_tail(DirectDevice &dd, int slot, uint32_t *flag, uin
     if (slot < 0 || slot >= kMaxDirectQueues || kernarg == nullptr || !direct_queue(dd, slot, &dq)) {
         return XCCL_ERR_NO_RESOURCE;
     }
-    if (dd.tail_kernel.object == 0) {
+    if (__atomic_load_n(&dd.tail_kernel.object, __ATOMIC_ACQUIRE) == 0) {
         std::lock_guard<std::mutex> guard(dd.lock);
         if (dd.tail_kernel.object == 0) {
             hsa_executable_symbol_t sym;
@@ -538,7 +540,8 @@ xccl_status_t direct_launch_tail(DirectDevice &dd, int slot, uint32_t *flag, uin
             if (kernarg_bytes > 16 || priv != 0 || k.object == 0) {
                 return XCCL_ERR_NO_RESOURCE;
             }
-            dd.tail_kernel = k;
+            dd.tail_kernel.group = k.group;
+            __atomic_store_n(&dd.tail_kernel.object, k.object, __ATOMIC_RELEASE);
         }
     }
     struct {
