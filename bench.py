@@ -65,9 +65,6 @@ def parse():
     ap.add_argument("--no-configs", action="store_true", help="skip the other benchmark configurations")
     ap.add_argument("--latency-iters", type=int, default=10000)
     ap.add_argument("--latency-quick", action="store_true", help="3 of the 14 message sizes only")
-    ap.add_argument("--one-thread", action="store_true",
-                    help="leave out the rows whose calls come from host threads started for them (in this process and in the "
-                         "child process): for runs under a profiler that interposes on queue submission")
     ap.add_argument("--profile-mode", nargs="?", const="headline", default=None,
                     choices=("headline", "footprint", "config3_int8", "config4_f16", "config4_f64", "small"),
                     help="for rocprofv3: only K launches of the named workload (headline: followed by K launches of a "
@@ -289,13 +286,13 @@ def latency_with_runtime_queues_in_device_memory(iters):
     return res
 
 
-def latency_extras(mc, hip, buf, iters, thread_counts=(1, 2, 4)):
+def latency_extras(mc, hip, buf, iters):
     from xccl_amd.types import Dt, Op, Status
     res = {}
     # blocking calls from several host threads at once (XCCL_THREAD_MODE_MULTIPLE, reference test/test_mt.c):
     # 4 sources x 1 KiB, every thread on operands of its own
     tb = hip.DeviceBuffer(8 * 8192)
-    for th in thread_counts:
+    for th in (1, 2, 4):
         st, ns = mc.bench_latency_mt(th, 8192, tb.ptr, tb.ptr + 1024, tb.ptr + 4096, 3, 256, 1024, Dt.FLOAT32, Op.SUM,
                                      iters)
         assert st == Status.OK
@@ -739,11 +736,10 @@ def main():
 
     if not a.no_latency:
         lat, lbuf = latency_sweep(mc, hip, a.latency_iters, a.latency_quick)
-        lat.update(latency_extras(mc, hip, lbuf, min(a.latency_iters, 4000), () if a.one_thread else (1, 2, 4)))
+        lat.update(latency_extras(mc, hip, lbuf, min(a.latency_iters, 4000)))
         lbuf.close()
-        if not a.one_thread:
-            lat["runtime_queue_rings_in_device_memory"] = latency_with_runtime_queues_in_device_memory(
-                min(a.latency_iters, 4000))
+        lat["runtime_queue_rings_in_device_memory"] = latency_with_runtime_queues_in_device_memory(
+            min(a.latency_iters, 4000))
         out["latency_us"] = lat
         out["mid_sizes"] = mid_sizes(mc, hip)
 

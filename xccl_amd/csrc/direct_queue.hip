@@ -72,6 +72,27 @@ struct DirectKernel {
 struct DirectQueue {
     hsa_queue_t *q       = nullptr;
     char        *kernarg = nullptr; // kKernargSlots slots, pinned host memory
+    // One producer at a time, from reserving a packet to ringing the doorbell for it.  The hardware queue would
+    // take packets from several producers at once, but a tool that interposes on queue submission (a profiler's
+    // intercept queue) then meets several new packets behind one doorbell, possibly across the ring's wrap; with
+    // one producer at a time every doorbell stands for exactly one new packet, in index order.  The section is a
+    // 64-byte store and a doorbell write.
+    std::atomic_flag turn = ATOMIC_FLAG_INIT;
+};
+
+struct QueueTurn {
+    explicit QueueTurn(DirectQueue &dq) : dq_(dq)
+    {
+        while (dq_.turn.test_and_set(std::memory_order_acquire)) {
+#if defined(__x86_64__) || defined(__i386__)
+            _mm_pause();
+#endif
+        }
+    }
+    ~QueueTurn() { dq_.turn.clear(std::memory_order_release); }
+    QueueTurn(const QueueTurn &)            = delete;
+    QueueTurn &operator=(const QueueTurn &) = delete;
+    DirectQueue &dq_;
 };
 
 struct DirectDevice {
@@ -468,6 +489,19 @@ xccl_status_t direct_launch(DirectDevice &dd, int slot, const Plan &plan, uint64
         return XCCL_ERR_NO_RESOURCE;
     }
 
+    if (kernarg != nullptr) {
+        // the caller's own argument block (its until the launch is complete).  It may be device memory behind a
+        // write-combining mapping: its stores leave the core before the doorbell's does (posted writes to one
+        // device arrive in order)
+        memcpy(kernarg, &plan.args, sizeof(ReduceArgs));
+#if defined(__x86_64__) || defined(__i386__)
+        _mm_sfence();
+#else
+        __atomic_thread_fence(__ATOMIC_SEQ_CST);
+#endif
+    }
+
+    QueueTurn      turn(*dq);
     hsa_queue_t   *q   = dq->q;
     const uint64_t idx = hsa_queue_add_write_index_scacq_screl(q, 1);
     while (idx - hsa_queue_load_read_index_scacquire(q) >= q->size) {
@@ -476,17 +510,10 @@ xccl_status_t direct_launch(DirectDevice &dd, int slot, const Plan &plan, uint64
             return XCCL_ERR_NO_RESOURCE; // the queue is dead; the reserved packet stays invalid
         }
     }
-    // the caller's own argument block (its until the launch is complete), else the queue's ring
-    char *args = kernarg != nullptr ? static_cast<char *>(kernarg) : dq->kernarg + (idx & (kKernargSlots - 1)) * kKernargSlot;
-    memcpy(args, &plan.args, sizeof(ReduceArgs));
-    if (kernarg != nullptr) {
-        // the block may be device memory behind a write-combining mapping: its stores leave the core before the
-        // doorbell's does (posted writes to one device arrive in order)
-#if defined(__x86_64__) || defined(__i386__)
-        _mm_sfence();
-#else
-        __atomic_thread_fence(__ATOMIC_SEQ_CST);
-#endif
+    char *args = static_cast<char *>(kernarg);
+    if (args == nullptr) {
+        args = dq->kernarg + (idx & (kKernargSlots - 1)) * kKernargSlot; // the queue's own ring of argument blocks
+        memcpy(args, &plan.args, sizeof(ReduceArgs));
     }
 
     hsa_kernel_dispatch_packet_t *p = static_cast<hsa_kernel_dispatch_packet_t *>(q->base_address) + (idx & (q->size - 1));
@@ -554,6 +581,7 @@ xccl_status_t direct_launch_tail(DirectDevice &dd, int slot, uint32_t *flag, uin
 #else
     __atomic_thread_fence(__ATOMIC_SEQ_CST);
 #endif
+    QueueTurn      turn(*dq);
     hsa_queue_t   *q   = dq->q;
     const uint64_t idx = hsa_queue_add_write_index_scacq_screl(q, 1);
     while (idx - hsa_queue_load_read_index_scacquire(q) >= q->size) {
@@ -585,41 +613,45 @@ xccl_status_t direct_launch_tail(DirectDevice &dd, int slot, uint32_t *flag, uin
     return XCCL_OK;
 }
 
-// Waits until everything queued on `q` has completed: a barrier packet with a
+// Waits until everything queued on `dq` has completed: a barrier packet with a
 // completion signal goes in behind it (a stream-ordered launch whose event
 // nobody waited for may still be queued or running when the component closes).
 // Bounded: gives up after `limit_ns`, or when the queue has reported an error.
-void direct_drain(hsa_queue_t *q, uint64_t limit_ns)
+void direct_drain(DirectQueue &dq, uint64_t limit_ns)
 {
+    hsa_queue_t *q = dq.q;
     hsa_signal_t done{};
     if (g_direct_failed.load(std::memory_order_acquire) != 0 ||
         hsa_amd_signal_create(1, 0, nullptr, HSA_AMD_SIGNAL_AMD_GPU_ONLY, &done) != HSA_STATUS_SUCCESS) {
         return;
     }
-    const uint64_t t0  = clock_ns();
-    const uint64_t idx = hsa_queue_add_write_index_scacq_screl(q, 1);
+    const uint64_t t0   = clock_ns();
     bool           room = true;
-    while (idx - hsa_queue_load_read_index_scacquire(q) >= q->size) {
-        if (g_direct_failed.load(std::memory_order_acquire) != 0 || clock_ns() - t0 > limit_ns) {
-            room = false; // the reserved packet stays invalid; the queue is about to be destroyed anyway
-            break;
-        }
-    }
-    if (room) {
-        hsa_barrier_and_packet_t *b = static_cast<hsa_barrier_and_packet_t *>(q->base_address) + (idx & (q->size - 1));
-        memset(reinterpret_cast<char *>(b) + 4, 0, sizeof(*b) - 4);
-        b->completion_signal = done;
-        const uint32_t header = (uint32_t)HSA_PACKET_TYPE_BARRIER_AND << HSA_PACKET_HEADER_TYPE |
-                                1u << HSA_PACKET_HEADER_BARRIER |
-                                (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE |
-                                (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE;
-        __atomic_store_n(reinterpret_cast<uint32_t *>(b), header, __ATOMIC_RELEASE);
-        hsa_signal_store_screlease(q->doorbell_signal, (hsa_signal_value_t)idx);
-        while (hsa_signal_load_scacquire(done) != 0) {
+    {
+        QueueTurn      turn(dq);
+        const uint64_t idx = hsa_queue_add_write_index_scacq_screl(q, 1);
+        while (idx - hsa_queue_load_read_index_scacquire(q) >= q->size) {
             if (g_direct_failed.load(std::memory_order_acquire) != 0 || clock_ns() - t0 > limit_ns) {
-                fprintf(stderr, "xccl mc_rocm: the component's dispatch queue did not drain; destroying it anyway\n");
+                room = false; // the reserved packet stays invalid; the queue is about to be destroyed anyway
                 break;
             }
+        }
+        if (room) {
+            hsa_barrier_and_packet_t *b = static_cast<hsa_barrier_and_packet_t *>(q->base_address) + (idx & (q->size - 1));
+            memset(reinterpret_cast<char *>(b) + 4, 0, sizeof(*b) - 4);
+            b->completion_signal = done;
+            const uint32_t header = (uint32_t)HSA_PACKET_TYPE_BARRIER_AND << HSA_PACKET_HEADER_TYPE |
+                                    1u << HSA_PACKET_HEADER_BARRIER |
+                                    (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCACQUIRE_FENCE_SCOPE |
+                                    (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE;
+            __atomic_store_n(reinterpret_cast<uint32_t *>(b), header, __ATOMIC_RELEASE);
+            hsa_signal_store_screlease(q->doorbell_signal, (hsa_signal_value_t)idx);
+        }
+    }
+    while (room && hsa_signal_load_scacquire(done) != 0) {
+        if (g_direct_failed.load(std::memory_order_acquire) != 0 || clock_ns() - t0 > limit_ns) {
+            fprintf(stderr, "xccl mc_rocm: the component's dispatch queue did not drain; destroying it anyway\n");
+            break;
         }
     }
     (void)hsa_signal_destroy(done);
@@ -632,7 +664,7 @@ void direct_destroy(DirectDevice &dd)
     std::lock_guard<std::mutex> guard(dd.lock);
     for (DirectQueue &dq : dd.queue) {
         if (dq.q != nullptr) {
-            direct_drain(dq.q, 10000000000ull);
+            direct_drain(dq, 10000000000ull);
             (void)hsa_queue_destroy(dq.q);
             dq.q = nullptr;
         }
@@ -761,7 +793,7 @@ xccl_status_t xccl_rocm_reduce_multi_direct(void *sbuf1, void *sbuf2, void *rbuf
             // store the word from here (it is host memory, at the same address on both sides)
             DirectQueue *dq = nullptr;
             if (direct_queue(*dd, queue_slot, &dq)) {
-                direct_drain(dq->q, 10000000000ull);
+                direct_drain(*dq, 10000000000ull);
             }
             __atomic_store_n(dev_flag, seq, __ATOMIC_RELEASE);
         }
