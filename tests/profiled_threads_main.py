@@ -16,6 +16,7 @@ from xccl_amd.types import Dt, MemType, Op, Status  # noqa: E402
 
 def main() -> int:
     threads, iters = 4, int(sys.argv[1]) if len(sys.argv) > 1 else 2000
+    print("started", flush=True)
     assert mc.xccl_mem_component_init() == Status.OK
     pitch = 8192
     buf = hip.DeviceBuffer(threads * pitch)
