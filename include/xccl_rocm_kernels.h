@@ -199,8 +199,9 @@ int xccl_rocm_direct_signal_done(uint64_t signal);
  *                   0 (default): they go to the HIP stream
  *                   (XCCL_MC_ROCM_DIRECT_SIGNAL)
  * Measured with the kernel arguments still in pinned host memory (in device
- * memory every row is 0.8 us lower and the shipped setting gives 4.6 / 4.8,
- * 5.3-5.5 / 5.7-6.0, 5.5-5.9 / 6.2-6.5), blocking call, 4 sources x 1 KiB,
+ * memory, with the flush write of xccl_rocm_set_direct_confirm, every row is
+ * 0.5 us lower and the shipped setting gives 4.8 / 5.0-6.1, 5.7 / 6.2-7.3,
+ * 6.0 / 6.6-8.0), blocking call, 4 sources x 1 KiB,
  * p50 / p99 in us, 1 / 2 / 4
  * calling threads: two queues shared, no barrier 5.5 / 5.8, 6.3 / 8.7,
  * 6.7-7.2 / 13.2; shared, with barrier 6.3 / 7.1, 6.1-6.4 / 8.8, 6.9-7.7 /
@@ -225,6 +226,19 @@ void xccl_rocm_set_direct_options(int acquire_system, int queues, int share,
  * 16.6, x 16 MiB 26.4 / 28.8 / 27.7, x 64 MiB 93.5 / 95.8 / 94.6, x 256 MiB
  * 353.7 / 357.8 / 355.2; 2 sources x 8 MiB 7.7 / 9.7 / 8.8. */
 void xccl_rocm_set_direct_tail(int on);
+
+/* What the host does between writing an argument block that lies in device
+ * memory and ringing the doorbell.  Host stores into device memory pass
+ * through the GPU's host data path, which may hold them back until it is
+ * flushed.  1 (default): write the device's flush register
+ * (HSA_AMD_AGENT_INFO_HDP_FLUSH), a posted write that arrives behind the
+ * argument stores and ahead of the doorbell; 2: also read that register back
+ * (returns when the flush is done); 3: read the block's last word back
+ * instead (returns when the stores are in device memory); 0: nothing but a
+ * store fence.  Measured per small call: 0: 4.6 us, 1: 4.9, 2: 6.0, 3: 6.3,
+ * blocks in pinned host memory (XCCL_MC_ROCM_DEVICE_KERNARG=0): 5.4.  Also
+ * XCCL_MC_ROCM_DIRECT_CONFIRM. */
+void xccl_rocm_set_direct_confirm(int mode);
 
 /* Launches that went out on the component's own queues so far (all devices). */
 uint64_t xccl_rocm_direct_launch_count(void);

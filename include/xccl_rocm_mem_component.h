@@ -106,7 +106,7 @@ extern "C" {
  *                    calls without an event; a call that has an event goes out
  *                    on a dispatch queue of the component's own instead when
  *                    the stream holds nothing it would have to stay behind
- *                    (4.4-5.6 us per small call instead of 6.8-7.7;
+ *                    (4.6-6.0 us per small call instead of 6.8-7.8;
  *                    XCCL_MC_ROCM_DIRECT_QUEUE=0 switches that off).  The
  *                    order of one thread's calls holds across the two; only
  *                    the event tells when such a call is complete.  Threads

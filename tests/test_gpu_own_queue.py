@@ -300,11 +300,18 @@ def test_kernel_arguments_in_device_memory_and_in_pinned_memory():
     """Launches on the own queues read their arguments from device memory that
     the host writes through the PCIe aperture (one arena per device, the same
     memory on every request that fits, none for a larger one); with
-    XCCL_MC_ROCM_DEVICE_KERNARG=0 they read them from pinned host memory.  Both
-    ways: 200 blocking calls on the own queue, results as numpy's."""
-    for env, arena in (({}, "True True True"), ({"XCCL_MC_ROCM_DEVICE_KERNARG": "0"}, "False True True")):
+    XCCL_MC_ROCM_DEVICE_KERNARG=0 they read them from pinned host memory.  Between
+    writing such a block and the doorbell the host writes the device's
+    host-data-path flush register (default), also reads it back, reads the
+    block back, or does neither (XCCL_MC_ROCM_DIRECT_CONFIRM = 1, 2, 3, 0).
+    Every way: 200 blocking calls on the own queue, results as numpy's."""
+    for env, arena in (({}, "True True True"), ({"XCCL_MC_ROCM_DEVICE_KERNARG": "0"}, "False True True"),
+                       ({"XCCL_MC_ROCM_DIRECT_CONFIRM": "0"}, "True True True"),
+                       ({"XCCL_MC_ROCM_DIRECT_CONFIRM": "2"}, "True True True"),
+                       ({"XCCL_MC_ROCM_DIRECT_CONFIRM": "3"}, "True True True")):
         e = dict(os.environ)
         e.pop("XCCL_MC_ROCM_DEVICE_KERNARG", None)
+        e.pop("XCCL_MC_ROCM_DIRECT_CONFIRM", None)
         e.update(env)
         out = subprocess.run([sys.executable, "-c", KERNARG_PROBE % ROOT], env=e, capture_output=True, text=True, timeout=120)
         assert out.returncode == 0, out.stdout + out.stderr

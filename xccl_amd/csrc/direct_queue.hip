@@ -40,8 +40,8 @@ namespace {
 //   Two queues per device by default, shared by the component's four thread
 // slots (slot s uses queue s mod 2), each created when a thread that uses it
 // first calls, behind that slot's HIP stream.  Measured with the argument
-// blocks in pinned host memory (in device memory every figure is 0.7-1 us
-// lower, and four threads see 5.5-5.9 / 6.2-6.5), blocking call, 4
+// blocks in pinned host memory (in device memory, flush write included, every
+// figure is about 0.5 us lower, and four threads see 6.0 / 6.6-8.0), blocking call, 4
 // sources x 1 KiB, p50 / p99 in us, 1 / 2 / 4 calling threads: this 5.5 / 5.8,
 // 6.3 / 8.7, 6.7-7.2 / 13.2; with the barrier bit on every packet 6.3 / 7.1,
 // 6.1-6.4 / 8.8, 6.9-7.7 / 13.6; slots 2 and 3 on HIP streams instead 5.4 / 5.8,
@@ -76,7 +76,7 @@ struct DirectQueue {
     // take packets from several producers at once, but a tool that interposes on queue submission (a profiler's
     // intercept queue) then meets several new packets behind one doorbell, possibly across the ring's wrap; with
     // one producer at a time every doorbell stands for exactly one new packet, in index order.  The section is a
-    // 64-byte store and a doorbell write.
+    // 64-byte store, the flush write for an argument block in device memory, and a doorbell write.
     std::atomic_flag turn = ATOMIC_FLAG_INIT;
 };
 
@@ -113,6 +113,7 @@ struct DirectDevice {
     // empty kernel's completion word is seen 3.7 us after the doorbell instead of 4.55).  Allocated once per
     // device and kept until the process ends, whatever happens to the queues.
     void                                         *arena       = nullptr;
+    volatile uint32_t                            *hdp_flush   = nullptr; // the device's host-data-path flush register
     size_t                                        arena_bytes = 0;
     bool                                          arena_tried = false;
 };
@@ -140,6 +141,65 @@ std::atomic<int>      g_direct_signal{0};
 //   g_direct_tail     1: such launches stay on the own queue with a one-lane kernel as a second packet behind
 //                     them that stores the completion word (XCCL_MC_ROCM_DIRECT_TAIL)
 std::atomic<int>      g_direct_tail{1};
+//   g_direct_confirm  what the host does between writing an argument block in device memory and ringing the
+//                     doorbell, see before_doorbell (XCCL_MC_ROCM_DIRECT_CONFIRM, 0..3)
+std::atomic<int>      g_direct_confirm{1};
+
+// Host stores into device memory pass through the GPU's host data path, which may hold them back; the runtime
+// names a register that, written, makes it pass them on (HSA_AMD_AGENT_INFO_HDP_FLUSH; the kernel driver and the
+// HIP runtime write it after their own stores into device memory).  After an argument block in device memory has
+// been written, before the doorbell:
+//   mode 1  the stores leave the core (sfence), then that register is written: a posted write that reaches the
+//           device behind the argument stores and ahead of the doorbell (default; +0.33 us per launch, measured)
+//   mode 2  the same, and the register is read back, which returns when the flush has been carried out (+1.4 us)
+//   mode 3  the block's last word is read back instead, which returns when the stores are in device memory
+//           (+1.3-1.7 us)
+//   mode 0  only the sfence (what the figures before this register was used were measured with: no stale
+//           argument in some 10^7 launches, but nothing says the host data path may not hold a store back)
+// Modes 2 and 3 cost more than keeping the blocks in pinned host memory (XCCL_MC_ROCM_DEVICE_KERNARG=0, +0.55 us).
+inline void store_fence()
+{
+#if defined(__x86_64__) || defined(__i386__)
+    _mm_sfence();
+#else
+    __atomic_thread_fence(__ATOMIC_SEQ_CST);
+#endif
+}
+
+// The last step before the doorbell of a launch whose argument block (`block`, `bytes`) lies in device memory and
+// has been written and fenced.  It comes behind the packet's own stores, so that it also covers a packet ring that
+// the runtime keeps in device memory (HSA_ALLOCATE_QUEUE_DEV_MEM=1).
+inline void before_doorbell(volatile uint32_t *hdp_flush, const void *block, size_t bytes)
+{
+    int mode = g_direct_confirm.load(std::memory_order_relaxed);
+    if (mode == 0) {
+        return;
+    }
+    if (hdp_flush == nullptr) {
+        mode = 3; // no such register on this device: the read-back is what is left
+    }
+    store_fence(); // the packet's stores too, should they be write-combined stores into device memory
+    if (mode == 1 || mode == 2) {
+        *hdp_flush = 1u;
+        if (mode == 2) {
+            (void)*hdp_flush;
+        }
+    } else {
+#if defined(__x86_64__) || defined(__i386__)
+        _mm_mfence();
+#endif
+        (void)*reinterpret_cast<const volatile uint32_t *>(static_cast<const char *>(block) + bytes - 4);
+    }
+#if defined(__x86_64__) || defined(__i386__)
+    if (mode == 1) {
+        _mm_sfence();
+    } else {
+        _mm_mfence();
+    }
+#else
+    __atomic_thread_fence(__ATOMIC_SEQ_CST);
+#endif
+}
 
 bool direct_enabled()
 {
@@ -154,6 +214,10 @@ bool direct_enabled()
         const char *t = getenv("XCCL_MC_ROCM_DIRECT_TAIL");
         if (t != nullptr) {
             g_direct_tail.store(atoi(t) != 0, std::memory_order_release);
+        }
+        const char *c = getenv("XCCL_MC_ROCM_DIRECT_CONFIRM");
+        if (c != nullptr) {
+            g_direct_confirm.store(atoi(c) < 0 || atoi(c) > 3 ? 1 : atoi(c), std::memory_order_release);
         }
         if (a != nullptr) {
             g_direct_acquire.store(strcmp(a, "system") == 0 ? HSA_FENCE_SCOPE_SYSTEM : HSA_FENCE_SCOPE_AGENT,
@@ -449,6 +513,10 @@ void *direct_arena(DirectDevice &dd, size_t bytes)
         return nullptr;
     }
     w[0] = 0;
+    hsa_amd_hdp_flush_t hdp{};
+    if (hsa_agent_get_info(dd.agent, (hsa_agent_info_t)HSA_AMD_AGENT_INFO_HDP_FLUSH, &hdp) == HSA_STATUS_SUCCESS) {
+        dd.hdp_flush = hdp.HDP_MEM_FLUSH_CNTL;
+    }
     dd.arena       = p;
     dd.arena_bytes = bytes;
     return p;
@@ -467,6 +535,14 @@ bool direct_signal_create(DirectDevice &dd, uint64_t *handle)
     dd.signals.push_back(sig);
     *handle = sig.handle;
     return true;
+}
+
+// Whether `p` lies in the device's arena of host-written device memory.
+inline bool in_arena(const DirectDevice &dd, const void *p)
+{
+    const char *c = static_cast<const char *>(p);
+    const char *a = static_cast<const char *>(dd.arena);
+    return a != nullptr && c >= a && c < a + dd.arena_bytes;
 }
 
 // Puts `plan` on queue `slot` of the current device.  `signal` != 0: the packet
@@ -494,11 +570,7 @@ xccl_status_t direct_launch(DirectDevice &dd, int slot, const Plan &plan, uint64
         // write-combining mapping: its stores leave the core before the doorbell's does (posted writes to one
         // device arrive in order)
         memcpy(kernarg, &plan.args, sizeof(ReduceArgs));
-#if defined(__x86_64__) || defined(__i386__)
-        _mm_sfence();
-#else
-        __atomic_thread_fence(__ATOMIC_SEQ_CST);
-#endif
+        store_fence();
     }
 
     QueueTurn      turn(*dq);
@@ -540,6 +612,9 @@ xccl_status_t direct_launch(DirectDevice &dd, int slot, const Plan &plan, uint64
     const uint32_t setup  = 1u << HSA_KERNEL_DISPATCH_PACKET_SETUP_DIMENSIONS;
     // header and setup share the packet's first 32-bit word: one release store makes the packet valid
     __atomic_store_n(reinterpret_cast<uint32_t *>(p), header | setup << 16, __ATOMIC_RELEASE);
+    if (in_arena(dd, kernarg)) {
+        before_doorbell(dd.hdp_flush, kernarg, sizeof(ReduceArgs));
+    }
     hsa_signal_store_screlease(q->doorbell_signal, (hsa_signal_value_t)idx);
     g_direct_launches.fetch_add(1, std::memory_order_relaxed);
     return XCCL_OK;
@@ -576,11 +651,7 @@ xccl_status_t direct_launch_tail(DirectDevice &dd, int slot, uint32_t *flag, uin
         uint32_t  seq, pad;
     } args = {flag, seq, 0};
     memcpy(kernarg, &args, sizeof(args));
-#if defined(__x86_64__) || defined(__i386__)
-    _mm_sfence();
-#else
-    __atomic_thread_fence(__ATOMIC_SEQ_CST);
-#endif
+    store_fence();
     QueueTurn      turn(*dq);
     hsa_queue_t   *q   = dq->q;
     const uint64_t idx = hsa_queue_add_write_index_scacq_screl(q, 1);
@@ -609,6 +680,9 @@ xccl_status_t direct_launch_tail(DirectDevice &dd, int slot, uint32_t *flag, uin
                             (uint32_t)HSA_FENCE_SCOPE_AGENT << HSA_PACKET_HEADER_SCRELEASE_FENCE_SCOPE;
     const uint32_t setup  = 1u << HSA_KERNEL_DISPATCH_PACKET_SETUP_DIMENSIONS;
     __atomic_store_n(reinterpret_cast<uint32_t *>(p), header | setup << 16, __ATOMIC_RELEASE);
+    if (in_arena(dd, kernarg)) {
+        before_doorbell(dd.hdp_flush, kernarg, sizeof(args));
+    }
     hsa_signal_store_screlease(q->doorbell_signal, (hsa_signal_value_t)idx);
     return XCCL_OK;
 }
@@ -821,6 +895,12 @@ int xccl_rocm_direct_signal_done(uint64_t signal)
 {
     return hsa_signal_load_scacquire(hsa_signal_t{signal}) == 0;
 }
+void xccl_rocm_set_direct_confirm(int on)
+{
+    (void)direct_enabled();
+    g_direct_confirm.store(on < 0 || on > 3 ? 1 : on, std::memory_order_release);
+}
+
 void xccl_rocm_set_direct_tail(int on)
 {
     (void)direct_enabled();

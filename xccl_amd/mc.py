@@ -108,6 +108,8 @@ def component_lib():
         lib.xccl_rocm_set_counted_grid.restype = None
         lib.xccl_rocm_set_direct_tail.argtypes = [_int]
         lib.xccl_rocm_set_direct_tail.restype = None
+        lib.xccl_rocm_set_direct_confirm.argtypes = [_int]
+        lib.xccl_rocm_set_direct_confirm.restype = None
         lib.xccl_rocm_set_direct_options.argtypes = [_int] * 5
         lib.xccl_rocm_set_direct_options.restype = None
         lib.xccl_rocm_set_slot_max_grid.argtypes = [_int]
